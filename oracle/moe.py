@@ -1,0 +1,149 @@
+"""CPU oracle: ragged expert GEMM, swiglu, k-way combine and the whole MoE FFN layer.
+
+Test infrastructure only.  Follows
+  * `apply_precision` + `matmul_torch`   python/triton_kernels/triton_kernels/matmul.py:772-931
+  * `swiglu_torch`                       .../swiglu.py:89-100   (evaluated in fp32 as the kernel does,
+                                         .../swiglu_details/_swiglu.py:55-64)
+  * `reduce_torch`                       .../reduce.py:1181-1214 (sum over `dim` in fp32, cast back)
+  * layer composition                    python/triton_kernels/tests/test_distributed.py:203-220 and
+                                         python/triton_kernels/bench/bench_mlp.py:60-96
+"""
+from __future__ import annotations
+
+import torch
+
+from . import mxfp as _mx
+from . import routing as _rt
+
+
+def dequant_weight(w: torch.Tensor, w_mx_scale: torch.Tensor | None, w_col_scale: torch.Tensor | None = None):
+    """Weights as the GEMM oracle multiplies them.
+
+    MX weights are dequantised to bf16 along K = dim -2 (matmul.py:799-811); plain weights are
+    used as stored (matmul.py:776-779).  `w_col_scale [E, N]` is the per-output-channel fp32
+    scale of the fp8 configuration, applied in fp32 (not pinned by the reference).
+    """
+    if w_mx_scale is not None:
+        w = _mx.upcast_from_mxfp(w, w_mx_scale, torch.bfloat16, axis=w.ndim - 2)
+    w = w.to("cpu")
+    if w_col_scale is not None:
+        w = w.to(torch.float32) * w_col_scale.to("cpu").to(torch.float32)[:, None, :]
+    return w
+
+
+def matmul(x, w, bias, slice_sizes=None, gather_indx=None, scatter_indx=None, gammas=None, betas=None,
+           w_mx_scale=None, x_row_scale=None, w_col_scale=None, out_dtype=None):
+    """Y[dst(r)] = cast(((X[src(r)] @ W[e(r)]) + bias[e(r)]*beta_r) * gamma_r)   (matmul.py:840-931).
+
+    `x [M,K]`; `w [E,K,N]` (or `[K,N]`); `slice_sizes [E]` rows per expert in sorted order (None: one
+    slice covering every row); accumulation in fp32 via `torch.matmul`; the result is rounded to
+    `out_dtype` (default: x's dtype, matmul.py:913-917) before the scatter; rows not written by the
+    scatter are zero (matmul.py:923-927).
+    """
+    x = x.detach().to("cpu")
+    w = dequant_weight(w, w_mx_scale, w_col_scale)
+    if w.ndim == 2:
+        w = w[None]
+    out_dtype = out_dtype or (x.dtype if x.dtype.itemsize > 1 else torch.bfloat16)
+    xf = x.to(torch.float32)
+    if x_row_scale is not None:
+        xf = xf * x_row_scale.to("cpu").to(torch.float32)[:, None]
+    n_rows = x.shape[0] if gather_indx is None else gather_indx.shape[0]
+    if slice_sizes is None:
+        bounds = [(0, n_rows)] * w.shape[0]
+        assert w.shape[0] == 1
+    else:
+        sizes = slice_sizes.detach().to("cpu").to(torch.int64)
+        off = torch.zeros(sizes.shape[0] + 1, dtype=torch.int64)
+        off[1:] = torch.cumsum(sizes, 0)
+        bounds = [(int(off[i]), int(off[i + 1])) for i in range(sizes.shape[0])]
+    N = w.shape[-1]
+    y = torch.zeros((n_rows, N), dtype=out_dtype)
+    gi = None if gather_indx is None else gather_indx.detach().to("cpu").to(torch.int64)
+    for e, (lo, hi) in enumerate(bounds):
+        if hi <= lo:
+            continue
+        idx = torch.arange(lo, hi) if gi is None else gi[lo:hi]
+        acc = torch.matmul(xf[idx, :], w[e].to(torch.float32))
+        if bias is not None:
+            b = bias.detach().to("cpu").to(torch.float32)
+            b = b[e] if b.ndim == 2 else b
+            acc += b if betas is None else b[None, :] * betas.to("cpu").to(torch.float32)[lo:hi, None]
+        if gammas is not None:
+            acc *= gammas.detach().to("cpu").to(torch.float32)[lo:hi, None]
+        y[lo:hi, :] = acc.to(out_dtype)
+    if scatter_indx is None:
+        return y
+    si = scatter_indx.detach().to("cpu").to(torch.int64)
+    out = torch.zeros((si.shape[0], N), dtype=out_dtype)
+    msk = si != -1
+    out[si[msk], :] = y[msk, :]
+    return out
+
+
+def swiglu(a: torch.Tensor, alpha: float, limit: float | None, out_dtype=None):
+    """Interleaved (gate, linear) columns -> s*(linear+1), s = g*sigmoid(alpha*g)   (swiglu.py:89-100)."""
+    a = a.detach().to("cpu")
+    out_dtype = out_dtype or a.dtype
+    af = a.to(torch.float32)
+    g = af[..., ::2]
+    l = af[..., 1::2]
+    if limit is not None:
+        g = g.clamp(max=limit)
+        l = l.clamp(min=-limit, max=limit)
+    s = g * torch.sigmoid(alpha * g)
+    return (s * (l + 1)).to(out_dtype)
+
+
+def reduce_k(y: torch.Tensor, k: int, mask: torch.Tensor | None = None):
+    """`[T*k, d] -> [T, d]`: sum of each token's k rows in fp32, cast back (reduce.py:1196-1203)."""
+    y = y.detach().to("cpu")
+    v = y.view(y.shape[0] // k, k, y.shape[-1]).to(torch.float32)
+    if mask is not None:
+        v = torch.where(mask.to("cpu").to(torch.bool), v, torch.zeros_like(v))
+    return v.sum(dim=1).to(y.dtype)
+
+
+def quantize_fp8_rowwise(x: torch.Tensor):
+    """Per-row dynamic e4m3 quantisation: `s = amax/448`, `q = sat_cast(x / s)`.
+
+    PARITY UNPINNED by the reference (no reference function computes it); follows the
+    saturating-cast note of mxfp.py:293-296.  An all-zero row gets scale 1 so it dequantises to 0.
+    """
+    xf = x.detach().to("cpu").to(torch.float32)
+    amax = xf.abs().amax(dim=-1)
+    s = amax / 448.0
+    s = torch.where(s == 0, torch.ones_like(s), s)
+    q = (xf / s[:, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return q, s
+
+
+def moe_layer(x, logits, k, w1, b1, w2, b2, swiglu_alpha=1.702, swiglu_limit=7.0, w1_mx_scale=None,
+              w2_mx_scale=None, w1_col_scale=None, w2_col_scale=None, fp8_activations=False,
+              return_intermediates=False):
+    """router -> gather-GEMM(+bias) -> swiglu -> scatter-GEMM(+bias, *gate) -> k-way sum.
+
+    Intermediates are rounded to bf16 exactly where the reference materialises them: `h` after the
+    first GEMM's epilogue (before swiglu, tests/test_matmul.py:622-623), the swiglu output, the
+    k-expanded `y`, and the combined output.
+    """
+    r = _rt.routing(logits, k, apply_softmax=True)
+    sizes = r.meta.col_sum
+    if fp8_activations:
+        xq, sx = quantize_fp8_rowwise(x)
+        h = matmul(xq, w1, b1, sizes, gather_indx=r.gather_indx, x_row_scale=sx, w_col_scale=w1_col_scale,
+                   out_dtype=torch.bfloat16)
+    else:
+        h = matmul(x, w1, b1, sizes, gather_indx=r.gather_indx, w_mx_scale=w1_mx_scale, w_col_scale=w1_col_scale)
+    a = swiglu(h, swiglu_alpha, swiglu_limit)
+    if fp8_activations:
+        aq, sa = quantize_fp8_rowwise(a)
+        y = matmul(aq, w2, b2, sizes, scatter_indx=r.scatter_indx, gammas=r.gammas, x_row_scale=sa,
+                   w_col_scale=w2_col_scale, out_dtype=torch.bfloat16)
+    else:
+        y = matmul(a, w2, b2, sizes, scatter_indx=r.scatter_indx, gammas=r.gammas, w_mx_scale=w2_mx_scale,
+                   w_col_scale=w2_col_scale)
+    out = reduce_k(y, k)
+    if return_intermediates:
+        return out, dict(routing=r, h=h, a=a, y=y)
+    return out

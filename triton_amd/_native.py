@@ -1,0 +1,104 @@
+"""ctypes binding of `libtriton_amd.so` (the C ABI declared in include/triton_amd.h).
+
+The library is loaded lazily on first use and a missing library is a hard error: there is no
+fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtriton_amd.so")
+
+TK_OK, TK_ERR_INVALID, TK_ERR_UNSUPPORTED, TK_ERR_LAUNCH = 0, 1, 2, 3
+
+# enum tk_dtype
+TK_F32, TK_BF16, TK_F16, TK_E4M3, TK_E5M2, TK_E2M1, TK_U8, TK_I16, TK_I32 = range(9)
+
+TORCH_TO_TK = {
+    torch.float32: TK_F32,
+    torch.bfloat16: TK_BF16,
+    torch.float16: TK_F16,
+    torch.float8_e4m3fn: TK_E4M3,
+    torch.float8_e5m2: TK_E5M2,
+    torch.uint8: TK_U8,
+    torch.int16: TK_I16,
+    torch.int32: TK_I32,
+}
+
+_c = ctypes
+_i32, _i64, _ptr, _f32 = _c.c_int32, _c.c_int64, _c.c_void_p, _c.c_float
+
+# name -> (restype, argtypes); must list every symbol include/triton_amd.h declares.
+SIGNATURES = {
+    "tk_version": (_i32, []),
+    "tk_last_error": (_c.c_char_p, []),
+    "tk_mx_downcast": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _i32, _i32, _ptr]),
+    "tk_mx_upcast": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i32, _i64, _i64, _i64, _ptr]),
+}
+
+# host-side check hooks (not part of the device ABI)
+HOST_SIGNATURES = {
+    "tk_host_mx_convert": (_i32, [_ptr, _i64, _i32, _ptr]),
+    "tk_host_mx_scale": (_i32, [_ptr, _i64, _i32, _i32, _ptr]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class NativeLibraryMissing(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded library; raises NativeLibraryMissing when it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise NativeLibraryMissing(
+                        f"{LIB_PATH} not found: build it with `python -m triton_amd.build` (needs hipcc). "
+                        "There is no fallback implementation.")
+                handle = ctypes.CDLL(LIB_PATH)
+                for name, (res, args) in {**SIGNATURES, **HOST_SIGNATURES}.items():
+                    fn = getattr(handle, name)
+                    fn.restype = res
+                    fn.argtypes = args
+                _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().tk_last_error().decode("utf-8", "replace")
+
+
+def check(status: int, what: str = ""):
+    """Maps a status code of the C ABI to the exception the reference raises in the same situation."""
+    if status == TK_OK:
+        return
+    msg = last_error() or what
+    if status == TK_ERR_INVALID:
+        raise ValueError(msg)
+    if status == TK_ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)
+
+
+def stream_ptr(device=None) -> int:
+    """The current PyTorch HIP stream of `device` as a raw hipStream_t."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor, name: str = "tensor"):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on a HIP device (got {t.device}); this package has no CPU path")
+
+
+def ptr(t) -> int | None:
+    return None if t is None else t.data_ptr()

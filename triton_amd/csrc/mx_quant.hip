@@ -1,0 +1,386 @@
+// MX quantise / dequantise kernels for gfx950 (HBM-bound byte work).
+//
+// Two source layouts are handled without a transposed temporary:
+//   rows : the quantised axis is the unit-stride one; 4 lanes share a block of 32, each holds 8
+//          consecutive elements, the block maximum is a 2-step lane exchange.
+//   cols : the quantised axis is strided and the INNER axis is unit-stride (a weight [E, K, N]
+//          quantised along K); a lane owns one or two columns and walks 32 rows, so every load of a
+//          wave is one contiguous row segment and the 32-element reduction is register-local.
+#include "mx_math.h"
+
+namespace tk {
+namespace {
+
+constexpr int kThreads = 256;
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<TK_F32> {
+  typedef float T;
+  static __device__ float load(const T* p) { return *p; }
+  static __device__ void store(T* p, float v) { *p = v; }
+  static __device__ float max_finite() { return 3.4028234663852886e+38f; }
+};
+template <>
+struct Elem<TK_BF16> {
+  typedef uint16_t T;
+  static __device__ float load(const T* p) { return bf16_bits_to_f32(*p); }
+  static __device__ void store(T* p, float v) { *p = f32_to_bf16_bits(v); }
+  static __device__ float max_finite() { return 3.3895313892515355e+38f; }
+};
+template <>
+struct Elem<TK_F16> {
+  typedef uint16_t T;
+  static __device__ float load(const T* p) { return f16_bits_to_f32(*p); }
+  static __device__ void store(T* p, float v) { *p = f32_to_f16_bits(v); }
+  static __device__ float max_finite() { return 65504.0f; }
+};
+
+// Index of the output line (run of one (outer, inner) coordinate along the quantised axis).  The inner
+// extent is mid x last with `last` fastest in the source; outputs order lines (outer, last, mid), which
+// is the order `x.transpose(axis, -1)` gives them.
+__device__ inline int64_t line_of(int64_t o, int64_t col, int64_t inner, int64_t inner_last) {
+  if (inner_last == inner) return o * inner + col;
+  const int64_t m = col / inner_last;
+  const int64_t l = col - m * inner_last;
+  return (o * inner_last + l) * (inner / inner_last) + m;
+}
+
+template <int KIND>
+__device__ inline uint32_t quant_byte(float q) {
+  if (KIND == TK_E4M3) return e4m3_byte(mx_clamp(q, 448.0f));
+  return e5m2_byte(mx_clamp(q, 57344.0f));
+}
+
+template <int KIND>
+__device__ inline float elem_f32(uint32_t b) {
+  if (KIND == TK_E4M3) return e4m3_to_f32(b);
+  return e5m2_to_f32(b);
+}
+
+// ---------------------------------------------------------------------------------------------
+// downcast, quantised axis contiguous: src [rows, L] with row stride `ld`
+// ---------------------------------------------------------------------------------------------
+template <int SRC, int KIND>
+__global__ __launch_bounds__(kThreads) void mx_down_rows(const typename Elem<SRC>::T* __restrict__ src, int64_t ld,
+                                                         int64_t rows, int64_t L, uint8_t* __restrict__ out_vals,
+                                                         uint8_t* __restrict__ out_scales, int rounding) {
+  const int64_t groups_per_row = L / 8;
+  const int64_t total = rows * groups_per_row;
+  const int64_t gid = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (gid >= total) return;  // total % 4 == 0, so a quad of lanes is either fully in or fully out
+  const int64_t row = gid / groups_per_row;
+  const int64_t g = gid - row * groups_per_row;
+  const typename Elem<SRC>::T* p = src + row * ld + g * 8;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = Elem<SRC>::load(p + i);
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) m = fmaxf(m, fabsf(v[i]));
+  m = fmaxf(m, __shfl_xor(m, 1));
+  m = fmaxf(m, __shfl_xor(m, 2));
+  const uint32_t sbits = mx_scale_bits(m, KIND, rounding);
+  const float inv = mx_inv_scale(sbits);
+  if (KIND == TK_E2M1) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) packed |= e2m1_code(v[i] * inv) << (4 * i);
+    *reinterpret_cast<uint32_t*>(out_vals + row * (L / 2) + g * 4) = packed;
+  } else {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lo |= quant_byte<KIND>(v[i] * inv) << (8 * i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hi |= quant_byte<KIND>(v[4 + i] * inv) << (8 * i);
+    *reinterpret_cast<uint2*>(out_vals + row * L + g * 8) = make_uint2(lo, hi);
+  }
+  if ((g & 3) == 0) out_scales[row * (L / 32) + (g >> 2)] = (uint8_t)(sbits >> 23);
+}
+
+// ---------------------------------------------------------------------------------------------
+// downcast, inner axis contiguous: src [outer, L, inner], stride_inner == 1
+// tile = 4 blocks of 32 rows x (64*CPT) columns per 256-thread workgroup; wave w owns block w
+// ---------------------------------------------------------------------------------------------
+template <int SRC, int KIND, int CPT>
+__global__ __launch_bounds__(kThreads) void mx_down_cols(const typename Elem<SRC>::T* __restrict__ src,
+                                                         int64_t stride_outer, int64_t stride_axis, int64_t L,
+                                                         int64_t inner, int64_t inner_last, int64_t col_tiles,
+                                                         int64_t blk_tiles, uint8_t* __restrict__ out_vals,
+                                                         uint8_t* __restrict__ out_scales, int rounding) {
+  typedef typename Elem<SRC>::T T;
+  int64_t bid = blockIdx.x;
+  const int64_t ct = bid % col_tiles;
+  bid /= col_tiles;
+  const int64_t bt = bid % blk_tiles;
+  const int64_t o = bid / blk_tiles;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t blk = bt * 4 + wave;
+  const int64_t col = (ct * 64 + lane) * CPT;
+  if (blk >= L / 32 || col >= inner) return;
+  const T* p = src + o * stride_outer + blk * 32 * stride_axis + col;
+  float v[32][CPT];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    if (CPT == 2) {
+      if (sizeof(T) == 2) {
+        uint32_t w = *reinterpret_cast<const uint32_t*>(p + i * stride_axis);
+        uint16_t a = (uint16_t)(w & 0xFFFFu), b = (uint16_t)(w >> 16);
+        v[i][0] = Elem<SRC>::load(reinterpret_cast<const T*>(&a));
+        v[i][CPT - 1] = Elem<SRC>::load(reinterpret_cast<const T*>(&b));
+      } else {
+        float2 w = *reinterpret_cast<const float2*>(p + i * stride_axis);
+        v[i][0] = w.x;
+        v[i][CPT - 1] = w.y;
+      }
+    } else {
+      v[i][0] = Elem<SRC>::load(p + i * stride_axis);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(v[i][c]));
+    const uint32_t sbits = mx_scale_bits(m, KIND, rounding);
+    const float inv = mx_inv_scale(sbits);
+    const int64_t line = line_of(o, col + c, inner, inner_last);
+    if (KIND == TK_E2M1) {
+      uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 32; ++i) w[i >> 3] |= e2m1_code(v[i][c] * inv) << (4 * (i & 7));
+      *reinterpret_cast<uint4*>(out_vals + line * (L / 2) + blk * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+      uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 32; ++i) w[i >> 2] |= quant_byte<KIND>(v[i][c] * inv) << (8 * (i & 3));
+      uint4* dst = reinterpret_cast<uint4*>(out_vals + line * L + blk * 32);
+      dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+      dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+    out_scales[line * (L / 32) + blk] = (uint8_t)(sbits >> 23);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// upcast, quantised axis contiguous in the output: out [rows, L] with row stride `ld`
+// ---------------------------------------------------------------------------------------------
+template <int KIND, int DST>
+__global__ __launch_bounds__(kThreads) void mx_up_rows(const uint8_t* __restrict__ vals,
+                                                       const uint8_t* __restrict__ scales, int64_t rows, int64_t L,
+                                                       typename Elem<DST>::T* __restrict__ out, int64_t ld) {
+  const int64_t groups_per_row = L / 8;
+  const int64_t total = rows * groups_per_row;
+  const int64_t gid = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (gid >= total) return;
+  const int64_t row = gid / groups_per_row;
+  const int64_t g = gid - row * groups_per_row;
+  const uint32_t sb = scales[row * (L / 32) + (g >> 2)];
+  const float mf = Elem<DST>::max_finite();
+  float v[8];
+  if (KIND == TK_E2M1) {
+    const uint32_t packed = *reinterpret_cast<const uint32_t*>(vals + row * (L / 2) + g * 4);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      v[i] = mx_dequant(bf16_bits_to_f32((uint16_t)e2m1_to_bf16_bits((packed >> (4 * i)) & 0xFu)), sb, mf, false);
+  } else {
+    const uint2 w = *reinterpret_cast<const uint2*>(vals + row * L + g * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = mx_dequant(elem_f32<KIND>((w.x >> (8 * i)) & 0xFFu), sb, mf, KIND == TK_E5M2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      v[4 + i] = mx_dequant(elem_f32<KIND>((w.y >> (8 * i)) & 0xFFu), sb, mf, KIND == TK_E5M2);
+  }
+  typename Elem<DST>::T* q = out + row * ld + g * 8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) Elem<DST>::store(q + i, v[i]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// upcast, inner axis contiguous in the output: out [outer, L, inner], ostride_inner == 1
+// ---------------------------------------------------------------------------------------------
+template <int KIND, int DST, int CPT>
+__global__ __launch_bounds__(kThreads) void mx_up_cols(const uint8_t* __restrict__ vals,
+                                                       const uint8_t* __restrict__ scales, int64_t L, int64_t inner,
+                                                       int64_t inner_last, int64_t col_tiles, int64_t blk_tiles,
+                                                       typename Elem<DST>::T* __restrict__ out,
+                                                       int64_t ostride_outer, int64_t ostride_axis) {
+  typedef typename Elem<DST>::T T;
+  int64_t bid = blockIdx.x;
+  const int64_t ct = bid % col_tiles;
+  bid /= col_tiles;
+  const int64_t bt = bid % blk_tiles;
+  const int64_t o = bid / blk_tiles;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t blk = bt * 4 + wave;
+  const int64_t col = (ct * 64 + lane) * CPT;
+  if (blk >= L / 32 || col >= inner) return;
+  const float mf = Elem<DST>::max_finite();
+  float v[32][CPT];
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int64_t line = line_of(o, col + c, inner, inner_last);
+    const uint32_t sb = scales[line * (L / 32) + blk];
+    if (KIND == TK_E2M1) {
+      const uint4 w4 = *reinterpret_cast<const uint4*>(vals + line * (L / 2) + blk * 16);
+      const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        v[i][c] = mx_dequant(bf16_bits_to_f32((uint16_t)e2m1_to_bf16_bits((w[i >> 3] >> (4 * (i & 7))) & 0xFu)), sb,
+                             mf, false);
+    } else {
+      const uint4* src = reinterpret_cast<const uint4*>(vals + line * L + blk * 32);
+      const uint4 a = src[0], b = src[1];
+      const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+        v[i][c] = mx_dequant(elem_f32<KIND>((w[i >> 2] >> (8 * (i & 3))) & 0xFFu), sb, mf, KIND == TK_E5M2);
+    }
+  }
+  T* q = out + o * ostride_outer + blk * 32 * ostride_axis + col;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    if (CPT == 2 && sizeof(T) == 2) {
+      uint16_t a, b;
+      Elem<DST>::store(reinterpret_cast<T*>(&a), v[i][0]);
+      Elem<DST>::store(reinterpret_cast<T*>(&b), v[i][CPT - 1]);
+      *reinterpret_cast<uint32_t*>(q + i * ostride_axis) = (uint32_t)a | ((uint32_t)b << 16);
+    } else if (CPT == 2) {
+      *reinterpret_cast<float2*>(q + i * ostride_axis) = make_float2(v[i][0], v[i][CPT - 1]);
+    } else {
+      Elem<DST>::store(q + i * ostride_axis, v[i][0]);
+    }
+  }
+}
+
+// ---- dispatch helpers --------------------------------------------------------------------------
+template <int SRC, int KIND>
+int32_t launch_down(const void* src, int64_t outer, int64_t L, int64_t inner, int64_t inner_last, int64_t so, int64_t sa, int64_t si,
+                    void* out_vals, void* out_scales, int rounding, hipStream_t st) {
+  typedef typename Elem<SRC>::T T;
+  const T* s = static_cast<const T*>(src);
+  uint8_t* ov = static_cast<uint8_t*>(out_vals);
+  uint8_t* os = static_cast<uint8_t*>(out_scales);
+  if (inner == 1 && sa == 1) {
+    // rows = outer, row stride = so
+    const int64_t total = outer * (L / 8);
+    const int64_t grid = cdiv(total, kThreads);
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_down_rows<SRC, KIND>), dim3((unsigned)grid), dim3(kThreads), 0, st, s, so, outer, L, ov, os,
+                       rounding);
+    return check_launch("mx_down_rows");
+  }
+  if (si != 1 && inner != 1) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: inner stride must be 1");
+  const int64_t nblk = L / 32;
+  const int64_t blk_tiles = cdiv(nblk, 4);
+  const size_t esz = sizeof(T);
+  const bool pair_ok = inner % 2 == 0 && sa % 2 == 0 && so % 2 == 0 && (reinterpret_cast<uintptr_t>(src) % (2 * esz)) == 0;
+  if (pair_ok) {
+    const int64_t col_tiles = cdiv(inner, 128);
+    const int64_t grid = col_tiles * blk_tiles * outer;
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_down_cols<SRC, KIND, 2>), dim3((unsigned)grid), dim3(kThreads), 0, st, s, so, sa, L, inner,
+                       inner_last, col_tiles, blk_tiles, ov, os, rounding);
+  } else {
+    const int64_t col_tiles = cdiv(inner, 64);
+    const int64_t grid = col_tiles * blk_tiles * outer;
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_down_cols<SRC, KIND, 1>), dim3((unsigned)grid), dim3(kThreads), 0, st, s, so, sa, L, inner,
+                       inner_last, col_tiles, blk_tiles, ov, os, rounding);
+  }
+  return check_launch("mx_down_cols");
+}
+
+template <int KIND, int DST>
+int32_t launch_up(const void* vals, const void* scales, int64_t outer, int64_t L, int64_t inner, int64_t inner_last, void* out, int64_t oso,
+                  int64_t osa, int64_t osi, hipStream_t st) {
+  typedef typename Elem<DST>::T T;
+  const uint8_t* v = static_cast<const uint8_t*>(vals);
+  const uint8_t* s = static_cast<const uint8_t*>(scales);
+  T* o = static_cast<T*>(out);
+  if (inner == 1 && osa == 1) {
+    const int64_t total = outer * (L / 8);
+    const int64_t grid = cdiv(total, kThreads);
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_up_rows<KIND, DST>), dim3((unsigned)grid), dim3(kThreads), 0, st, v, s, outer, L, o, oso);
+    return check_launch("mx_up_rows");
+  }
+  if (osi != 1 && inner != 1) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: output inner stride must be 1");
+  const int64_t nblk = L / 32;
+  const int64_t blk_tiles = cdiv(nblk, 4);
+  const size_t esz = sizeof(T);
+  const bool pair_ok = inner % 2 == 0 && osa % 2 == 0 && oso % 2 == 0 && (reinterpret_cast<uintptr_t>(out) % (2 * esz)) == 0;
+  if (pair_ok) {
+    const int64_t col_tiles = cdiv(inner, 128);
+    const int64_t grid = col_tiles * blk_tiles * outer;
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_up_cols<KIND, DST, 2>), dim3((unsigned)grid), dim3(kThreads), 0, st, v, s, L, inner,
+                       inner_last, col_tiles, blk_tiles, o, oso, osa);
+  } else {
+    const int64_t col_tiles = cdiv(inner, 64);
+    const int64_t grid = col_tiles * blk_tiles * outer;
+    if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: tensor too large for one launch");
+    hipLaunchKernelGGL((mx_up_cols<KIND, DST, 1>), dim3((unsigned)grid), dim3(kThreads), 0, st, v, s, L, inner,
+                       inner_last, col_tiles, blk_tiles, o, oso, osa);
+  }
+  return check_launch("mx_up_cols");
+}
+
+}  // namespace
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int32_t tk_mx_downcast(const void* src, int32_t src_dtype, int64_t outer, int64_t axis_len, int64_t inner,
+                                  int64_t inner_last, int64_t stride_outer, int64_t stride_axis, int64_t stride_inner, void* out_vals,
+                                  void* out_scales, int32_t out_kind, int32_t rounding, tk_stream_t stream) {
+  if (outer < 0 || axis_len < 0 || inner < 0) return fail(TK_ERR_INVALID, "tk_mx_downcast: negative size");
+  if (axis_len % 32 != 0) return fail(TK_ERR_INVALID, "tk_mx_downcast: axis length %lld is not a multiple of 32", (long long)axis_len);
+  if (rounding != TK_MX_ROUND_UP && rounding != TK_MX_ROUND_DOWN) return fail(TK_ERR_INVALID, "tk_mx_downcast: bad rounding mode %d", rounding);
+  if (out_kind != TK_E2M1 && out_kind != TK_E4M3 && out_kind != TK_E5M2) return fail(TK_ERR_INVALID, "tk_mx_downcast: bad output kind %d", out_kind);
+  if (outer == 0 || axis_len == 0 || inner == 0) return TK_OK;
+  if (inner_last <= 0 || inner % inner_last != 0) return fail(TK_ERR_INVALID, "tk_mx_downcast: inner_last must divide inner");
+  if (!src || !out_vals || !out_scales) return fail(TK_ERR_INVALID, "tk_mx_downcast: null pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define TK_DOWN(S, K) \
+  if (src_dtype == S && out_kind == K) return launch_down<S, K>(src, outer, axis_len, inner, inner_last, stride_outer, stride_axis, stride_inner, out_vals, out_scales, rounding, st);
+  TK_DOWN(TK_BF16, TK_E2M1)
+  TK_DOWN(TK_BF16, TK_E4M3)
+  TK_DOWN(TK_BF16, TK_E5M2)
+  TK_DOWN(TK_F16, TK_E2M1)
+  TK_DOWN(TK_F16, TK_E4M3)
+  TK_DOWN(TK_F16, TK_E5M2)
+  TK_DOWN(TK_F32, TK_E2M1)
+  TK_DOWN(TK_F32, TK_E4M3)
+  TK_DOWN(TK_F32, TK_E5M2)
+#undef TK_DOWN
+  return fail(TK_ERR_INVALID, "tk_mx_downcast: unsupported source dtype %d", src_dtype);
+}
+
+extern "C" int32_t tk_mx_upcast(const void* vals, const void* scales, int32_t kind, int64_t outer, int64_t axis_len,
+                                int64_t inner, int64_t inner_last, void* out, int32_t out_dtype, int64_t ostride_outer,
+                                int64_t ostride_axis, int64_t ostride_inner, tk_stream_t stream) {
+  if (outer < 0 || axis_len < 0 || inner < 0) return fail(TK_ERR_INVALID, "tk_mx_upcast: negative size");
+  if (axis_len % 32 != 0) return fail(TK_ERR_INVALID, "tk_mx_upcast: axis length %lld is not a multiple of 32", (long long)axis_len);
+  if (kind != TK_E2M1 && kind != TK_E4M3 && kind != TK_E5M2) return fail(TK_ERR_INVALID, "tk_mx_upcast: bad element kind %d", kind);
+  if (outer == 0 || axis_len == 0 || inner == 0) return TK_OK;
+  if (inner_last <= 0 || inner % inner_last != 0) return fail(TK_ERR_INVALID, "tk_mx_upcast: inner_last must divide inner");
+  if (!vals || !scales || !out) return fail(TK_ERR_INVALID, "tk_mx_upcast: null pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define TK_UP(K, D) \
+  if (kind == K && out_dtype == D) return launch_up<K, D>(vals, scales, outer, axis_len, inner, inner_last, out, ostride_outer, ostride_axis, ostride_inner, st);
+  TK_UP(TK_E2M1, TK_BF16)
+  TK_UP(TK_E2M1, TK_F16)
+  TK_UP(TK_E2M1, TK_F32)
+  TK_UP(TK_E4M3, TK_BF16)
+  TK_UP(TK_E4M3, TK_F16)
+  TK_UP(TK_E4M3, TK_F32)
+  TK_UP(TK_E5M2, TK_BF16)
+  TK_UP(TK_E5M2, TK_F16)
+  TK_UP(TK_E5M2, TK_F32)
+#undef TK_UP
+  return fail(TK_ERR_INVALID, "tk_mx_upcast: unsupported output dtype %d", out_dtype);
+}
