@@ -99,6 +99,167 @@ int32_t tk_mx_upcast(const void* vals, const void* scales, int32_t kind, int64_t
                      int64_t inner, int64_t inner_last, void* out, int32_t out_dtype, int64_t ostride_outer, int64_t ostride_axis,
                      int64_t ostride_inner, tk_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Router: top-k (+softmax), expert histogram, gather/scatter permutations, ragged block schedule
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * One routing pass.  Replaces, in three launches, the reference's
+ *   `_topk_forward[(pids,)](...)`                          tk/topk.py:59-67
+ *   `_sum_bitmatrix_rows[(grid_m, grid_n)](...)`           tk/tensor_details/bitmatrix_details/sum_bitmatrix_rows.py:89-97
+ *   `_bitmatrix_metadata_compute_stage1/2[...]`            tk/tensor_details/bitmatrix.py:128-145
+ *   `_ragged_tensor_metadata_memset/compute[...]`          tk/tensor_details/ragged_tensor.py:197-208
+ * and the torch glue `gather = col_sorted // k`, `gammas = vals.flatten()[col_sorted]`
+ * (python/triton_kernels/tests/test_distributed.py:203-210).
+ *
+ * Selection is a stable descending sort: ties go to the lower expert id; outputs are ordered by value,
+ * largest first; the softmax runs over the k kept logits in fp32.  Rows >= n_rows are left untouched
+ * in vals / indx / bitmatrix and are not routed.  Optional outputs may be NULL; when col_sum is NULL
+ * only the top-k step runs.  Limits: n_experts <= 2048, k <= min(64, n_experts).
+ */
+typedef struct tk_route_desc {
+  const void* logits; /* [n_tokens, n_experts], unit stride along experts; may be NULL with use_provided_indx */
+  int32_t logits_dtype; /* TK_F32, TK_BF16, TK_F16 */
+  int64_t logits_stride_m;
+  int32_t n_tokens;
+  int32_t n_rows;            /* rows to route, -1 = all */
+  const int32_t* n_rows_ptr; /* device scalar overriding n_rows, or NULL */
+  int32_t n_experts;
+  int32_t k;
+  int32_t apply_softmax;
+  int32_t use_provided_indx; /* 1: `indx` is an input (tk/topk.py:121-123) */
+  void* vals;                /* out [n_tokens, k], logits dtype, or NULL */
+  void* indx;                /* [n_tokens, k] */
+  int32_t indx_dtype;        /* TK_I16 */
+  void* bitmatrix;           /* out uint32 [ceil(E/32)][bitmatrix_stride_w]: word w of token t at w*stride + t; or NULL */
+  int64_t bitmatrix_stride_w;
+  int32_t* col_sum;         /* out [n_experts] tokens per expert */
+  int32_t* col_sorted_indx; /* out [n_tokens*k] flat position t*k+j of each expert-sorted row, -1 padded */
+  int32_t* row_sorted_indx; /* out [n_tokens*k] inverse permutation, -1 padded */
+  int32_t* gather_indx;     /* out [n_tokens*k] token of each expert-sorted row (= col_sorted / k), or NULL */
+  void* gammas;             /* out [n_tokens*k] gate value of each expert-sorted row (logits dtype), or NULL */
+  /* ragged metadata of col_sum for block sizes 16, 32, 64, 128, 256 (all NULL to skip) */
+  int32_t* slice_offs;     /* out [n_experts + 1] */
+  int32_t* block_offs;     /* out [5][block_offs_stride], first n_experts + 1 entries of each row */
+  int64_t block_offs_stride;
+  int32_t* block_schedule; /* out [5][block_schedule_stride], first max_n_blocks entries of each row */
+  int64_t block_schedule_stride;
+  int32_t max_n_blocks;
+  void* workspace; /* tk_route_workspace_bytes(n_tokens, n_experts) bytes, needed when col_sum != NULL */
+} tk_route_desc;
+
+int64_t tk_route_workspace_bytes(int32_t n_tokens, int32_t n_experts);
+int32_t tk_route(const tk_route_desc* desc, tk_stream_t stream);
+
+/*
+ * Replaces `_ragged_tensor_metadata_memset` + `_ragged_tensor_metadata_compute`
+ * (tk/tensor_details/ragged_tensor.py:183-210): slice_offs = [0] + cumsum(slice_sizes); for block sizes
+ * 16..256: block_offs = [0] + cumsum(ceil(slice_sizes / bs)) and block_schedule[offs[s] + b] =
+ * (b << 16) | s, padded with -1 up to max_n_blocks.
+ */
+int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t* slice_offs, int32_t* block_offs,
+                           int64_t block_offs_stride, int32_t* block_schedule, int64_t block_schedule_stride,
+                           int32_t max_n_blocks, tk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Ragged expert GEMM
+ * ---------------------------------------------------------------------------------------------- */
+
+enum tk_activation {
+  TK_ACT_NONE = 0,
+  TK_ACT_SWIGLU = 1 /* interleaved (gate, linear) columns -> N/2 outputs, tk/swiglu_details/_swiglu.py:55-70 */
+};
+
+/*
+ * Operands of one ragged GEMM launch.  Plain data, filled by the host; pointers are device pointers,
+ * NULL means "absent".  Mirrors the argument list of the `_matmul[(grid,)](...)` launch of
+ * tk/matmul.py:659-726 restricted to what a mixture-of-experts forward uses.
+ *
+ *   Y[dst(r), :] = act( (X[src(r), :] @ W[e(r)]) * x_row_scale[src(r)] * w_col_scale[e(r), :]
+ *                        + bias[e(r), :] ) * gammas[r]
+ *
+ * r runs over rows in expert-sorted order; e(r) is the slice containing r; src(r) = gather_indx[r]
+ * (or r); dst(r) = scatter_indx[r] (or r), rows with dst(r) == -1 are not written.  Accumulation is
+ * fp32; the epilogue order is that of tk/matmul_details/_matmul.py:507-559.
+ */
+typedef struct tk_gemm_desc {
+  /* activations: [rows, K], unit stride along K */
+  const void* x;
+  int32_t x_dtype; /* TK_BF16, or TK_E4M3 with x_row_scale */
+  int64_t x_stride_m;
+  const float* x_row_scale; /* fp32 per ROW OF x (indexed after the gather), or NULL */
+  /* weights: [E, K, N]; e2m1 is packed two per byte along K and the strides count bytes */
+  const void* w;
+  int32_t w_dtype; /* TK_BF16, TK_E2M1 (needs w_mx_scale), TK_E4M3 */
+  int64_t w_stride_e, w_stride_k, w_stride_n;
+  const void* w_mx_scale; /* uint8 e8m0 [E, K/32, N] or NULL */
+  int64_t ws_stride_e, ws_stride_k, ws_stride_n;
+  const float* w_col_scale; /* fp32 [E, N] (unit stride along N) or NULL */
+  int64_t wcs_stride_e;
+  /* bias [E, N] (unit stride along N), fp32 or bf16 */
+  const void* bias;
+  int32_t bias_dtype;
+  int64_t bias_stride_e;
+  /* row indirection and per-row scale (expert-sorted order) */
+  const int32_t* gather_indx;
+  const int32_t* scatter_indx;
+  int32_t scatter_len;
+  const void* gammas;
+  int32_t gammas_dtype; /* TK_F32 or TK_BF16 */
+  /* ragged metadata for `block_m` (tk/tensor_details/ragged_tensor.py:12-94); all NULL = one slice of M rows */
+  const int32_t* slice_sizes;
+  const int32_t* slice_offs;
+  const int32_t* block_offs;     /* [n_slices + 1] for block_m */
+  const int32_t* block_schedule; /* [grid_m] for block_m, (block << 16) | slice, -1 padded */
+  int32_t n_slices;
+  int32_t block_m; /* 16, 32, 64 or 128 */
+  int32_t grid_m;  /* number of row blocks to launch (an upper bound in ragged mode) */
+  int32_t M, N, K; /* M: rows of the single slice when not ragged; N: columns of W; K: reduction */
+  /* output [rows, N or N/2], unit stride along N */
+  void* y;
+  int32_t y_dtype; /* TK_BF16 */
+  int64_t y_stride_m;
+  int32_t activation; /* enum tk_activation */
+  float act_alpha, act_limit;
+  int32_t act_has_limit;
+} tk_gemm_desc;
+
+/* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */
+int32_t tk_moe_gemm(const tk_gemm_desc* desc, tk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Element-wise companions of the GEMM
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * Standalone swiglu; replaces the `_swiglu[grid](...)` launch of tk/swiglu.py:56-79.
+ * a [M, 2*n_out] with interleaved (gate, linear) columns -> out [M, n_out], same dtype
+ * (TK_BF16 / TK_F16 / TK_F32), fp32 arithmetic.  n_rows_ptr (device scalar, may be NULL) bounds M.
+ */
+int32_t tk_swiglu(const void* a, int32_t dtype, int64_t M, int64_t n_out, int64_t stride_am, void* out,
+                  int64_t stride_om, float alpha, float limit, int32_t has_limit, const int32_t* n_rows_ptr,
+                  tk_stream_t stream);
+
+/*
+ * Sum over the middle dimension; replaces the `_reduce_forward[grid](...)` launch of tk/reduce.py:664-853
+ * for dim == 1 (the k-way combine of expert outputs).
+ * y[a, c] = sum_j (mask[a, j, c] ? x[a, j, c] * scale[a, j, c] : 0); x [A, K, C] with unit stride along C;
+ * mask (uint8/bool) and scale (fp32) are optional and addressed through their own strides (0 = broadcast);
+ * fp32 accumulation in j order; y has x's dtype.
+ */
+int32_t tk_reduce_mid(const void* x, int32_t dtype, int64_t A, int64_t K, int64_t C, int64_t sx0, int64_t sx1,
+                      const void* mask, int64_t sm0, int64_t sm1, int64_t sm2, const float* scale, int64_t ss0,
+                      int64_t ss1, int64_t ss2, void* y, int64_t sy0, tk_stream_t stream);
+
+/*
+ * Per-row dynamic quantisation of bf16 activations to OCP e4m3: scales[m] = amax_m / 448 (1 for a zero
+ * row), q[m, :] = saturating_cast(x[m, :] / scales[m]).  No counterpart kernel in the reference: its
+ * benchmark casts activations to fp8 with a plain torch `.to()` (python/triton_kernels/bench/bench_mlp.py:169);
+ * the scales feed tk_gemm_desc.x_row_scale.
+ */
+int32_t tk_quant_fp8_rows(const void* x, int32_t dtype, int64_t M, int64_t K, int64_t stride_m, void* q,
+                          int64_t stride_qm, float* scales, tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

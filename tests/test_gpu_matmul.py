@@ -1,0 +1,141 @@
+"""GPU parity of the ragged expert GEMM (through the C ABI) against the CPU oracle.
+
+Mirrors the gfx950-relevant slice of python/triton_kernels/tests/test_matmul.py:116-301: bf16 x bf16 and
+bf16 x mxfp4, plain and ragged (10 slices, one empty), x {none, gather, scatter, gather+scatter} x gammas,
+block_m in {16, 128}, fused swiglu.  Tolerances are the reference's (testing.py:27-88, test_matmul.py:644-653)
+and the rtol 2e-2 / atol 1e-2 gate."""
+import pytest
+import torch
+
+from oracle import moe as omoe
+from oracle import mxfp as omx
+from oracle import routing as ort
+from oracle.checks import assert_allclose_gate, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mods(device):
+    import triton_amd.matmul as mm
+    import triton_amd.swiglu as sw
+    import triton_amd.tensor as tensor
+    return mm, sw, tensor
+
+
+def _slice_sizes(m, n_slices, g):
+    cuts = torch.sort(torch.randint(0, m + 1, (n_slices - 1, ), generator=g)).values
+    sizes = torch.diff(torch.cat([torch.tensor([0]), cuts, torch.tensor([m])]))
+    if n_slices > 2:
+        sizes[n_slices // 2 + 1] += sizes[n_slices // 2]  # one empty slice (testing.py:307-311)
+        sizes[n_slices // 2] = 0
+    return sizes.to(torch.int32)
+
+
+def _make_w(E, K, N, kind, g, device):
+    w = (torch.randn((E, K, N), generator=g) * 0.5 / K**0.5 * 4).to(torch.bfloat16)
+    if kind == "mxfp4":
+        q, s = omx.downcast_to_mxfp(w, torch.uint8, axis=1)
+        return dict(w_dev=q.to(device), scale_dev=s.to(device), w_cpu=q, scale_cpu=s)
+    if kind == "bf16_kmajor":
+        wd = w.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)
+        return dict(w_dev=wd, scale_dev=None, w_cpu=w, scale_cpu=None)
+    return dict(w_dev=w.to(device), scale_dev=None, w_cpu=w, scale_cpu=None)
+
+
+CASES = [
+    # m, n, k, mode, wkind
+    (16, 256, 256, "ragged", "bf16"),
+    (300, 400, 400, "ragged", "bf16_kmajor"),
+    (300, 400, 416, "ragged", "mxfp4"),
+    (1000, 704, 832, "ragged", "bf16_kmajor"),
+    (720, 576, 768, "ragged", "mxfp4"),
+    (768, 512, 1024, "ragged", "mxfp4"),
+    (720, 576, 768, "plain", "mxfp4"),
+    (600, 400, 416, "plain", "bf16"),
+    (5, 2880, 2880, "ragged", "mxfp4"),
+]
+
+
+@pytest.mark.parametrize("m, n, k, mode, wkind", CASES)
+@pytest.mark.parametrize("block_m", [16, 128])
+@pytest.mark.parametrize("do_gather, do_scatter", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("do_gamma", [False, True])
+def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatter, do_gamma):
+    mm, _, tensor = mods
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + k + block_m)
+    n_slices = 10 if mode == "ragged" else 1
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, wkind, g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g) if mode == "ragged" else None
+    gather = torch.randint(0, m, (m, ), generator=g, dtype=torch.int32) if do_gather else None
+    scatter = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    if scatter is not None and m > 20:
+        scatter[torch.rand(m, generator=g) < 0.05] = -1
+    gammas = 2.0**torch.randint(-5, 0, (m, ), generator=g).float() if do_gamma else None
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m) if sizes is not None else None
+    pc = mm.PrecisionConfig(b_mx_scale=W["scale_dev"])
+    dev = lambda t: None if t is None else t.to(device)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(x.to(device), W["w_dev"], dev(bias) if mode == "ragged" else dev(bias[0]), md, gather_indx=dev(gather),
+                      scatter_indx=dev(scatter), precision_config=pc, gammas=dev(gammas))
+    ref = omoe.matmul(x, W["w_cpu"], bias, sizes, gather_indx=gather, scatter_indx=scatter, gammas=gammas,
+                      w_mx_scale=W["scale_cpu"])
+    got = y.cpu()
+    if scatter is not None:  # rows that no entry writes are undefined in the kernel path, zero in the oracle
+        written = torch.zeros(m, dtype=torch.bool)
+        written[scatter[scatter >= 0].long()] = True
+        got = torch.where(written[:, None], got, torch.zeros_like(got))
+    assert_close(ref, got, maxtol=3e-2 if wkind == "mxfp4" else 2e-2, what="y")
+    assert_allclose_gate(ref, got, what="y")
+
+
+@pytest.mark.parametrize("m, n, k, wkind", [(300, 512, 416, "bf16_kmajor"), (720, 576, 768, "mxfp4"), (40, 5760, 2880, "mxfp4")])
+@pytest.mark.parametrize("block_m", [16, 32, 64, 128])
+@pytest.mark.parametrize("opts", [(1.1, 1.4), (1.702, 7.0), (0.5, None)])
+def test_fused_swiglu(mods, device, m, n, k, wkind, block_m, opts):
+    mm, sw, tensor = mods
+    g = torch.Generator().manual_seed(m + n + k)
+    n_slices = 6
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, wkind, g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw.swiglu_fn, ("alpha", "limit"), reduction_n=2), opts)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]),
+                      fused_activation=act)
+    h = omoe.matmul(x, W["w_cpu"], bias, sizes, w_mx_scale=W["scale_cpu"])
+    ref = omoe.swiglu(h, opts[0], opts[1])
+    assert y.shape == (m, n // 2)
+    assert_close(ref, y, maxtol=3e-2, what="swiglu(y)")
+    # standalone swiglu kernel on the unfused GEMM output
+    y2 = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]))
+    s2 = sw.swiglu(y2, opts[0], sw.PrecisionConfig(opts[1]))
+    assert_close(omoe.swiglu(y2.cpu(), opts[0], opts[1]), s2, maxtol=1e-2, what="standalone swiglu")
+
+
+def test_zero_sized(mods, device):
+    mm, _, tensor = mods
+    for m, n, k in [(0, 5, 7), (5, 0, 7)]:
+        x = torch.zeros((m, k), dtype=torch.bfloat16, device=device)
+        w = torch.zeros((1, k, n), dtype=torch.bfloat16, device=device)
+        assert mm.matmul(x, w, None).shape == (m, n)
+
+
+def test_rejected_options(mods, device):
+    mm, _, _ = mods
+    x = torch.zeros((4, 32), dtype=torch.bfloat16, device=device)
+    w = torch.zeros((1, 32, 16), dtype=torch.bfloat16, device=device)
+    with pytest.raises(NotImplementedError):
+        mm.matmul(x, w, None, betas=torch.ones(4, device=device))
+    with pytest.raises(NotImplementedError):
+        mm.matmul(x, w, None, c_acc_in=torch.zeros((4, 16), device=device))
+    with pytest.raises(mm.InapplicableConstraint):
+        with mm.scoped_opt_flags_constraints({"split_k": 2}):
+            mm.matmul(x, w, None)
+    with pytest.raises(mm.InapplicableConstraint):
+        with mm.scoped_opt_flags_constraints({"is_persistent": True}):
+            mm.matmul(x, w, None)

@@ -33,11 +33,50 @@ TORCH_TO_TK = {
 _c = ctypes
 _i32, _i64, _ptr, _f32 = _c.c_int32, _c.c_int64, _c.c_void_p, _c.c_float
 
+TK_ACT_NONE, TK_ACT_SWIGLU = 0, 1
+
+
+class RouteDesc(_c.Structure):
+    """struct tk_route_desc (field order and types follow include/triton_amd.h)."""
+    _fields_ = [
+        ("logits", _ptr), ("logits_dtype", _i32), ("logits_stride_m", _i64), ("n_tokens", _i32), ("n_rows", _i32),
+        ("n_rows_ptr", _ptr), ("n_experts", _i32), ("k", _i32), ("apply_softmax", _i32), ("use_provided_indx", _i32),
+        ("vals", _ptr), ("indx", _ptr), ("indx_dtype", _i32), ("bitmatrix", _ptr), ("bitmatrix_stride_w", _i64),
+        ("col_sum", _ptr), ("col_sorted_indx", _ptr), ("row_sorted_indx", _ptr), ("gather_indx", _ptr),
+        ("gammas", _ptr), ("slice_offs", _ptr), ("block_offs", _ptr), ("block_offs_stride", _i64),
+        ("block_schedule", _ptr), ("block_schedule_stride", _i64), ("max_n_blocks", _i32), ("workspace", _ptr),
+    ]
+
+
+class GemmDesc(_c.Structure):
+    """struct tk_gemm_desc (field order and types follow include/triton_amd.h)."""
+    _fields_ = [
+        ("x", _ptr), ("x_dtype", _i32), ("x_stride_m", _i64), ("x_row_scale", _ptr),
+        ("w", _ptr), ("w_dtype", _i32), ("w_stride_e", _i64), ("w_stride_k", _i64), ("w_stride_n", _i64),
+        ("w_mx_scale", _ptr), ("ws_stride_e", _i64), ("ws_stride_k", _i64), ("ws_stride_n", _i64),
+        ("w_col_scale", _ptr), ("wcs_stride_e", _i64),
+        ("bias", _ptr), ("bias_dtype", _i32), ("bias_stride_e", _i64),
+        ("gather_indx", _ptr), ("scatter_indx", _ptr), ("scatter_len", _i32),
+        ("gammas", _ptr), ("gammas_dtype", _i32),
+        ("slice_sizes", _ptr), ("slice_offs", _ptr), ("block_offs", _ptr), ("block_schedule", _ptr),
+        ("n_slices", _i32), ("block_m", _i32), ("grid_m", _i32), ("M", _i32), ("N", _i32), ("K", _i32),
+        ("y", _ptr), ("y_dtype", _i32), ("y_stride_m", _i64),
+        ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
+    ]
+
+
 # name -> (restype, argtypes); must list every symbol include/triton_amd.h declares.
 SIGNATURES = {
     "tk_version": (_i32, []),
     "tk_last_error": (_c.c_char_p, []),
     "tk_mx_downcast": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _i32, _i32, _ptr]),
+    "tk_route_workspace_bytes": (_i64, [_i32, _i32]),
+    "tk_route": (_i32, [_c.POINTER(RouteDesc), _ptr]),
+    "tk_ragged_metadata": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _i64, _i32, _ptr]),
+    "tk_moe_gemm": (_i32, [_c.POINTER(GemmDesc), _ptr]),
+    "tk_swiglu": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _f32, _f32, _i32, _ptr, _ptr]),
+    "tk_reduce_mid": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
+    "tk_quant_fp8_rows": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
     "tk_mx_upcast": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i32, _i64, _i64, _i64, _ptr]),
 }
 

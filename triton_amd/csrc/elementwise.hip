@@ -1,0 +1,141 @@
+// Small HBM-bound kernels around the expert GEMMs: standalone swiglu, the k-way combine
+// (masked / scaled sum over the expert dimension) and per-row dynamic fp8 quantisation.
+#include "mx_math.h"
+
+namespace tk {
+namespace {
+
+template <int DT>
+__device__ inline float ld(const void* p, int64_t i) {
+  if (DT == TK_F32) return static_cast<const float*>(p)[i];
+  if (DT == TK_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+}
+template <int DT>
+__device__ inline void st(void* p, int64_t i, float v) {
+  if (DT == TK_F32)
+    static_cast<float*>(p)[i] = v;
+  else if (DT == TK_BF16)
+    static_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  else
+    static_cast<uint16_t*>(p)[i] = f32_to_f16_bits(v);
+}
+
+// out[m, j] = s * (l + 1), s = g * sigmoid(alpha * g), (g, l) = (a[m, 2j], a[m, 2j+1]) after clamping.
+template <int DT>
+__global__ __launch_bounds__(256) void swiglu_kernel(const void* a, int64_t stride_am, void* out, int64_t stride_om,
+                                                     int64_t M, int64_t N, float alpha, float limit, int has_limit,
+                                                     const int32_t* n_rows_ptr) {
+  if (n_rows_ptr) M = *n_rows_ptr < M ? *n_rows_ptr : M;
+  const int64_t total = M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / N, j = i - m * N;
+    float g = ld<DT>(a, m * stride_am + 2 * j);
+    float l = ld<DT>(a, m * stride_am + 2 * j + 1);
+    if (has_limit) {
+      g = fminf(g, limit);
+      l = fminf(fmaxf(l, -limit), limit);
+    }
+    const float s = g / (1.0f + expf(-alpha * g));
+    st<DT>(out, m * stride_om + j, fmaf(s, l, s));
+  }
+}
+
+// y[a, c] = sum_j mask[a, j, c] ? x[a, j, c] * scale[a, j, c] : 0, fp32 accumulation in j order.
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_mid_kernel(const void* x, int64_t sx0, int64_t sx1, int64_t A, int64_t K,
+                                                         int64_t C, const uint8_t* mask, int64_t sm0, int64_t sm1,
+                                                         int64_t sm2, const float* scale, int64_t ss0, int64_t ss1,
+                                                         int64_t ss2, void* y, int64_t sy0) {
+  const int64_t total = A * C;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t a = i / C, c = i - a * C;
+    float acc = 0.f;
+    for (int64_t j = 0; j < K; ++j) {
+      float v = ld<DT>(x, a * sx0 + j * sx1 + c);
+      if (scale) v *= scale[a * ss0 + j * ss1 + c * ss2];
+      if (mask && !mask[a * sm0 + j * sm1 + c * sm2]) v = 0.f;
+      acc += v;
+    }
+    st<DT>(y, a * sy0 + c, acc);
+  }
+}
+
+// Per-row dynamic quantisation to OCP e4m3: s = amax / 448 (1 for an all-zero row), q = sat(x / s).
+// One wave per row; the row is read twice (second pass hits L2).
+__global__ __launch_bounds__(256) void quant_fp8_rows_kernel(const uint16_t* x, int64_t stride_m, int64_t M, int64_t K,
+                                                             uint8_t* q, int64_t stride_qm, float* scales) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const uint16_t* xr = x + row * stride_m;
+  float m = 0.f;
+  for (int64_t k = lane; k < K; k += 64) m = fmaxf(m, fabsf(bf16_bits_to_f32(xr[k])));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  float s = m / 448.0f;
+  if (s == 0.f) s = 1.0f;
+  if (lane == 0) scales[row] = s;
+  uint8_t* qr = q + row * stride_qm;
+  for (int64_t k = lane; k < K; k += 64) qr[k] = (uint8_t)e4m3_byte(mx_clamp(bf16_bits_to_f32(xr[k]) / s, 448.0f));
+}
+
+int grid_for(int64_t total) {
+  int64_t g = cdiv(total, 256);
+  return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
+}
+
+}  // namespace
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int32_t tk_swiglu(const void* a, int32_t dtype, int64_t M, int64_t n_out, int64_t stride_am, void* out,
+                             int64_t stride_om, float alpha, float limit, int32_t has_limit, const int32_t* n_rows_ptr,
+                             tk_stream_t stream) {
+  if (M < 0 || n_out < 0) return fail(TK_ERR_INVALID, "tk_swiglu: negative size");
+  if (M == 0 || n_out == 0) return TK_OK;
+  if (!a || !out) return fail(TK_ERR_INVALID, "tk_swiglu: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int grid = grid_for(M * n_out);
+  if (dtype == TK_BF16)
+    hipLaunchKernelGGL(swiglu_kernel<TK_BF16>, dim3(grid), dim3(256), 0, s, a, stride_am, out, stride_om, M, n_out, alpha, limit, has_limit, n_rows_ptr);
+  else if (dtype == TK_F16)
+    hipLaunchKernelGGL(swiglu_kernel<TK_F16>, dim3(grid), dim3(256), 0, s, a, stride_am, out, stride_om, M, n_out, alpha, limit, has_limit, n_rows_ptr);
+  else if (dtype == TK_F32)
+    hipLaunchKernelGGL(swiglu_kernel<TK_F32>, dim3(grid), dim3(256), 0, s, a, stride_am, out, stride_om, M, n_out, alpha, limit, has_limit, n_rows_ptr);
+  else
+    return fail(TK_ERR_UNSUPPORTED, "tk_swiglu: dtype %d", dtype);
+  return check_launch("swiglu_kernel");
+}
+
+extern "C" int32_t tk_reduce_mid(const void* x, int32_t dtype, int64_t A, int64_t K, int64_t C, int64_t sx0, int64_t sx1,
+                                 const void* mask, int64_t sm0, int64_t sm1, int64_t sm2, const float* scale, int64_t ss0,
+                                 int64_t ss1, int64_t ss2, void* y, int64_t sy0, tk_stream_t stream) {
+  if (A < 0 || K < 0 || C < 0) return fail(TK_ERR_INVALID, "tk_reduce_mid: negative size");
+  if (A == 0 || C == 0) return TK_OK;
+  if (!x || !y) return fail(TK_ERR_INVALID, "tk_reduce_mid: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int grid = grid_for(A * C);
+  const uint8_t* m = static_cast<const uint8_t*>(mask);
+  if (dtype == TK_BF16)
+    hipLaunchKernelGGL(reduce_mid_kernel<TK_BF16>, dim3(grid), dim3(256), 0, s, x, sx0, sx1, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, y, sy0);
+  else if (dtype == TK_F16)
+    hipLaunchKernelGGL(reduce_mid_kernel<TK_F16>, dim3(grid), dim3(256), 0, s, x, sx0, sx1, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, y, sy0);
+  else if (dtype == TK_F32)
+    hipLaunchKernelGGL(reduce_mid_kernel<TK_F32>, dim3(grid), dim3(256), 0, s, x, sx0, sx1, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, y, sy0);
+  else
+    return fail(TK_ERR_UNSUPPORTED, "tk_reduce_mid: dtype %d", dtype);
+  return check_launch("reduce_mid_kernel");
+}
+
+extern "C" int32_t tk_quant_fp8_rows(const void* x, int32_t dtype, int64_t M, int64_t K, int64_t stride_m, void* q,
+                                     int64_t stride_qm, float* scales, tk_stream_t stream) {
+  if (M < 0 || K < 0) return fail(TK_ERR_INVALID, "tk_quant_fp8_rows: negative size");
+  if (M == 0) return TK_OK;
+  if (!x || !q || !scales) return fail(TK_ERR_INVALID, "tk_quant_fp8_rows: null pointer");
+  if (dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_quant_fp8_rows: input must be bf16");
+  hipLaunchKernelGGL(quant_fp8_rows_kernel, dim3((unsigned)cdiv(M, 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x), stride_m, M, K, static_cast<uint8_t*>(q), stride_qm, scales);
+  return check_launch("quant_fp8_rows_kernel");
+}

@@ -1,0 +1,488 @@
+// Top-k softmax router, expert histogram / gather-scatter indices and ragged block schedule for gfx950.
+//
+// The reference spends six dependent launches here (top-k, vertical popcount, two metadata stages,
+// two ragged-metadata kernels).  Here the work is three launches, all latency-bound integer work:
+//
+//   route_topk_kernel    one wave64 owns a run of `rows_per_wave` tokens.  A row's logits sit in
+//                        registers (lane l holds experts l, l+64, ...); each of the k rounds is a
+//                        wave-wide max-reduction of a 64-bit key (order-preserving float key in the high
+//                        word, ~expert in the low word, so ties go to the LOWER expert id).  The wave
+//                        also accumulates its private per-expert histogram in LDS and writes it out
+//                        as one row of `partials`.
+//   route_scan_kernel    ONE workgroup: per expert an exclusive prefix over the waves' histograms,
+//                        the expert totals (`col_sum`), their exclusive scan (`col_offs`) and, if
+//                        asked, the whole ragged metadata (slice offsets, block offsets and block
+//                        schedules for block sizes 16..256).
+//   route_scatter_kernel each wave re-reads its tokens' expert ids in flat (token-major) order, ranks
+//                        equal ids with ballots (stable), and writes both permutations plus the
+//                        optional gather index / gate value in expert-sorted order.
+#include "common.h"
+
+namespace tk {
+namespace {
+
+constexpr int kMaxExperts = 2048;  // per-wave LDS histogram: 4 waves x 2048 x 4 B = 32 KiB
+constexpr int kWaves = 4;
+constexpr int kNumBlockSizes = 5;  // 16, 32, 64, 128, 256
+constexpr int kFirstBlockLog2 = 4;
+
+__device__ inline uint32_t ordered_key(float v) {
+  const uint32_t u = f32_bits(v);
+  return u ^ ((u & 0x80000000u) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ inline float key_to_float(uint32_t k) {
+  return bits_f32(k ^ ((k & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu));
+}
+
+// Orders this wave's LDS accesses: lanes exchange data through LDS without a workgroup barrier.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ inline unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned long long o = __shfl_xor(v, off);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__device__ inline float wave_sum_f32(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+template <int DT>
+__device__ inline float load_logit(const void* p, int64_t i) {
+  if (DT == TK_F32) return static_cast<const float*>(p)[i];
+  if (DT == TK_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+}
+template <int DT>
+__device__ inline void store_val(void* p, int64_t i, float v) {
+  if (DT == TK_F32)
+    static_cast<float*>(p)[i] = v;
+  else if (DT == TK_BF16)
+    static_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  else
+    static_cast<uint16_t*>(p)[i] = f32_to_f16_bits(v);
+}
+
+struct TopkParams {
+  const void* logits;  // [T, E] or null (histogram of given indices only)
+  int64_t stride_m;
+  int32_t T;
+  int32_t n_rows_imm;
+  const int32_t* n_rows_ptr;
+  int32_t E, k;
+  int32_t apply_softmax;
+  int32_t use_provided_indx;
+  void* vals;               // [T, k] logits dtype, or null
+  int16_t* indx;            // [T, k]
+  uint32_t* bitmatrix;      // [words][T_pad] or null
+  int64_t bm_stride_w;
+  int32_t* partials;        // [units][E] or null
+  int32_t rows_per_wave;
+  int32_t* fill_a;          // [T*k] arrays preset to -1 (the two permutations and the gather index), or null
+  int32_t* fill_b;
+  int32_t* fill_c;
+};
+
+template <int DT, int EPL>
+__global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParams p) {
+  __shared__ int32_t hist_s[kWaves][EPL * 64];
+  __shared__ uint32_t words_s[kWaves][EPL * 2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x * kWaves + wave;
+  const int E = p.E, k = p.k;
+  const int n_rows = p.n_rows_ptr ? *p.n_rows_ptr : p.n_rows_imm;
+  const int words = (E + 31) / 32;
+  for (int e = lane; e < EPL * 64; e += 64) hist_s[wave][e] = 0;
+  const int row_begin = unit * p.rows_per_wave;
+  int row_end = row_begin + p.rows_per_wave;
+  row_end = row_end < p.T ? row_end : p.T;
+  if (p.fill_a) {
+    // entries that are never routed (masked rows, dropped indices) leave -1 in the permutations
+    for (int64_t f = (int64_t)row_begin * k + lane; f < (int64_t)row_end * k; f += 64) {
+      p.fill_a[f] = -1;
+      p.fill_b[f] = -1;
+      if (p.fill_c) p.fill_c[f] = -1;
+    }
+  }
+  for (int row = row_begin; row < row_end; ++row) {
+    if (row >= n_rows) break;
+    float myval = 0.f;
+    int myidx = -1;
+    if (p.use_provided_indx) {
+      if (lane < k) {
+        myidx = p.indx[(int64_t)row * k + lane];
+        if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
+      }
+    } else {
+      unsigned long long key[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        if (e < E) {
+          const float v = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e);
+          key[i] = ((unsigned long long)ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e);
+        } else {
+          key[i] = 0ull;
+        }
+      }
+      for (int j = 0; j < k; ++j) {
+        unsigned long long best = key[0];
+#pragma unroll
+        for (int i = 1; i < EPL; ++i) best = key[i] > best ? key[i] : best;
+        best = wave_max_u64(best);
+#pragma unroll
+        for (int i = 0; i < EPL; ++i)
+          if (key[i] == best) key[i] = 0ull;
+        if (lane == j) {
+          myval = key_to_float((uint32_t)(best >> 32));
+          myidx = (int)(~(uint32_t)best);
+        }
+      }
+    }
+    float outv = myval;
+    if (p.apply_softmax) {
+      // softmax over the k kept logits in fp32; the largest sits in lane 0
+      float vmax = myval;
+      if (p.use_provided_indx) {
+        float m = lane < k ? myval : -INFINITY;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+        vmax = m;
+      } else {
+        vmax = __shfl(myval, 0);
+      }
+      const float z = lane < k ? expf(myval - vmax) : 0.f;
+      const float sum = wave_sum_f32(z);
+      outv = z / sum;
+    }
+    if (lane < k) {
+      if (p.vals) store_val<DT>(p.vals, (int64_t)row * k + lane, outv);
+      if (!p.use_provided_indx) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
+    }
+    const bool live = lane < k && myidx >= 0 && myidx < E;
+    if (p.partials && live) atomicAdd(&hist_s[wave][myidx], 1);
+    if (p.bitmatrix) {
+      for (int w = lane; w < words; w += 64) words_s[wave][w] = 0u;
+      wave_sync();
+      if (live) atomicOr(&words_s[wave][myidx >> 5], 1u << (myidx & 31));
+      wave_sync();
+      for (int w = lane; w < words; w += 64) p.bitmatrix[(int64_t)w * p.bm_stride_w + row] = words_s[wave][w];
+      wave_sync();
+    }
+  }
+  if (p.partials && row_begin < p.T) {
+    wave_sync();
+    for (int e = lane; e < E; e += 64) p.partials[(int64_t)unit * E + e] = hist_s[wave][e];
+  }
+}
+
+// ---- block-wide exclusive scan (1024 threads) ---------------------------------------------------
+constexpr int kScanThreads = 1024;
+
+__device__ __forceinline__ int block_exclusive_scan(int v, int* total) {
+  __shared__ int wave_sums[kScanThreads / 64 + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(inc, off);
+    if (lane >= off) inc += o;
+  }
+  __syncthreads();  // protects wave_sums against the previous call's readers
+  if (lane == 63) wave_sums[wave] = inc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+      const int t = wave_sums[w];
+      wave_sums[w] = run;
+      run += t;
+    }
+    wave_sums[kScanThreads / 64] = run;
+  }
+  __syncthreads();
+  *total = wave_sums[kScanThreads / 64];
+  return inc - v + wave_sums[wave];
+}
+
+// out[i] = sum_{j<i} f(in[j]) for i in [0, n], f(x) = ceil(x / 2^shift)
+__device__ __forceinline__ void scan_to(const int32_t* in, int n, int shift, int32_t* out) {
+  int carry = 0;
+  for (int base = 0; base < n; base += kScanThreads) {
+    const int i = base + threadIdx.x;
+    int v = 0;
+    if (i < n) v = (in[i] + ((1 << shift) - 1)) >> shift;
+    int total;
+    const int ex = block_exclusive_scan(v, &total);
+    if (i < n) out[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) out[n] = carry;
+}
+
+struct RaggedOut {
+  int32_t* slice_offs;    // [E+1]
+  int32_t* block_offs;    // [kNumBlockSizes][stride]
+  int64_t block_offs_stride;
+  int32_t* block_sched;   // [kNumBlockSizes][stride]
+  int64_t block_sched_stride;
+  int32_t max_n_blocks;
+};
+
+__device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int E, const RaggedOut r) {
+  scan_to(slice_sizes, E, 0, r.slice_offs);
+  for (int b = 0; b < kNumBlockSizes; ++b)
+    scan_to(slice_sizes, E, kFirstBlockLog2 + b, r.block_offs + b * r.block_offs_stride);
+  for (int b = 0; b < kNumBlockSizes; ++b)
+    for (int i = threadIdx.x; i < r.max_n_blocks; i += kScanThreads) r.block_sched[b * r.block_sched_stride + i] = -1;
+  __threadfence_block();
+  __syncthreads();
+  for (int b = 0; b < kNumBlockSizes; ++b) {
+    const int shift = kFirstBlockLog2 + b;
+    const int32_t* offs = r.block_offs + b * r.block_offs_stride;
+    int32_t* sched = r.block_sched + b * r.block_sched_stride;
+    for (int e = threadIdx.x; e < E; e += kScanThreads) {
+      const int nb = (slice_sizes[e] + ((1 << shift) - 1)) >> shift;
+      const int o = offs[e];
+      for (int j = 0; j < nb; ++j)
+        if (o + j < r.max_n_blocks) sched[o + j] = (j << 16) | e;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* partials, int units, int E, int32_t* col_sum,
+                                                                  int32_t* col_offs, int want_ragged, const RaggedOut r) {
+  for (int e = threadIdx.x; e < E; e += kScanThreads) {
+    int run = 0;
+    for (int u = 0; u < units; ++u) {
+      const int64_t i = (int64_t)u * E + e;
+      const int t = partials[i];
+      partials[i] = run;
+      run += t;
+    }
+    col_sum[e] = run;
+  }
+  __threadfence_block();
+  __syncthreads();
+  scan_to(col_sum, E, 0, col_offs);
+  if (want_ragged) {
+    __threadfence_block();
+    __syncthreads();
+    ragged_metadata(col_sum, E, r);
+  }
+}
+
+__global__ __launch_bounds__(kScanThreads) void ragged_metadata_kernel(const int32_t* slice_sizes, int E, const RaggedOut r) {
+  ragged_metadata(slice_sizes, E, r);
+}
+
+struct ScatterParams {
+  const int16_t* indx16;  // [T, k] (one of indx16 / indx32)
+  const int32_t* indx32;
+  int32_t T, k, E;
+  int32_t n_rows_imm;
+  const int32_t* n_rows_ptr;
+  int32_t rows_per_wave;
+  const int32_t* partials;  // [units][E], exclusive over units
+  const int32_t* col_offs;  // [E+1]
+  int32_t* col_sorted;      // [T*k]
+  int32_t* row_sorted;      // [T*k]
+  int32_t* gather_out;      // [T*k] or null: token feeding sorted row
+  const void* vals;         // [T, k] or null
+  void* gammas_out;         // [T*k] or null: gate value of sorted row (same dtype as vals)
+  int32_t vals_bytes;       // 2 or 4
+};
+
+__global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const ScatterParams p) {
+  __shared__ int32_t base_s[kWaves][kMaxExperts];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x * kWaves + wave;
+  const int E = p.E, k = p.k;
+  const int n_rows = p.n_rows_ptr ? *p.n_rows_ptr : p.n_rows_imm;
+  const int row_begin = unit * p.rows_per_wave;
+  if (row_begin >= p.T) return;
+  int row_end = row_begin + p.rows_per_wave;
+  row_end = row_end < p.T ? row_end : p.T;
+  for (int e = lane; e < E; e += 64) base_s[wave][e] = p.col_offs[e] + p.partials[(int64_t)unit * E + e];
+  wave_sync();
+  const int64_t f_begin = (int64_t)row_begin * k, f_end = (int64_t)row_end * k;
+  const int64_t n_valid = (int64_t)(n_rows < p.T ? n_rows : p.T) * k;
+  const unsigned long long lt_mask = (1ull << lane) - 1ull;
+  for (int64_t f0 = f_begin; f0 < f_end; f0 += 64) {
+    const int64_t f = f0 + lane;
+    const bool in = f < f_end;
+    int e = -1;
+    if (in && f < n_valid) e = p.indx16 ? (int)p.indx16[f] : p.indx32[f];
+    const bool valid = e >= 0 && e < E;
+    int pos = -1;
+    unsigned long long todo = __ballot(valid);
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const int e0 = __shfl(e, leader);
+      const unsigned long long same = __ballot(valid && e == e0);
+      if (valid && e == e0) pos = base_s[wave][e0] + __popcll(same & lt_mask);
+      wave_sync();
+      if (lane == leader) base_s[wave][e0] = base_s[wave][e0] + __popcll(same);
+      wave_sync();
+      todo &= ~same;
+    }
+    if (valid) {
+      p.row_sorted[f] = pos;
+      p.col_sorted[pos] = (int32_t)f;
+      if (p.gather_out) p.gather_out[pos] = (int32_t)(f / k);
+      if (p.gammas_out) {
+        if (p.vals_bytes == 4)
+          static_cast<uint32_t*>(p.gammas_out)[pos] = static_cast<const uint32_t*>(p.vals)[f];
+        else
+          static_cast<uint16_t*>(p.gammas_out)[pos] = static_cast<const uint16_t*>(p.vals)[f];
+      }
+    }
+  }
+}
+
+int rows_per_wave_for(int T) {
+  int rpw = 16;
+  while ((int64_t)rpw * 1024 < T) rpw *= 2;
+  return rpw;
+}
+
+template <int DT>
+int32_t launch_topk(const TopkParams& p, int units, hipStream_t st) {
+  const int grid = (units + kWaves - 1) / kWaves;
+  const int epl = (p.E + 63) / 64;
+#define TK_EPL(N)                                                                                              \
+  if (epl <= N) {                                                                                              \
+    hipLaunchKernelGGL((route_topk_kernel<DT, N>), dim3(grid), dim3(kWaves * 64), 0, st, p);                    \
+    return check_launch("route_topk_kernel");                                                                  \
+  }
+  TK_EPL(1)
+  TK_EPL(2)
+  TK_EPL(4)
+  TK_EPL(8)
+  TK_EPL(16)
+  TK_EPL(32)
+#undef TK_EPL
+  return fail(TK_ERR_UNSUPPORTED, "tk_route: more than %d experts", kMaxExperts);
+}
+
+}  // namespace
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int64_t tk_route_workspace_bytes(int32_t T, int32_t E) {
+  if (T <= 0 || E <= 0) return 0;
+  const int rpw = rows_per_wave_for(T);
+  const int64_t units = (T + rpw - 1) / rpw;
+  const int64_t units_pad = (units + kWaves - 1) / kWaves * kWaves;
+  return (units_pad * E + (int64_t)E + 1) * 4;
+}
+
+extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
+  if (!d) return fail(TK_ERR_INVALID, "tk_route: null descriptor");
+  const int T = d->n_tokens, E = d->n_experts, k = d->k;
+  if (T < 0 || E <= 0 || k <= 0) return fail(TK_ERR_INVALID, "tk_route: bad sizes T=%d E=%d k=%d", T, E, k);
+  if (k > 64 || k > E) return fail(TK_ERR_INVALID, "tk_route: k=%d must be <= min(64, E)", k);
+  if (E > kMaxExperts) return fail(TK_ERR_UNSUPPORTED, "tk_route: at most %d experts are supported (got %d)", kMaxExperts, E);
+  if (T == 0) return TK_OK;
+  const bool want_meta = d->col_sum != nullptr;
+  if (!d->indx) return fail(TK_ERR_INVALID, "tk_route: indx buffer is required");
+  if (!d->logits && !d->use_provided_indx) return fail(TK_ERR_INVALID, "tk_route: logits are required unless indices are provided");
+  if (want_meta && (!d->col_sorted_indx || !d->row_sorted_indx || !d->workspace)) return fail(TK_ERR_INVALID, "tk_route: metadata outputs / workspace missing");
+  if (d->indx_dtype != TK_I16) return fail(TK_ERR_UNSUPPORTED, "tk_route: indx must be int16");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int rpw = rows_per_wave_for(T);
+  const int units = (T + rpw - 1) / rpw;
+  const int units_pad = (units + kWaves - 1) / kWaves * kWaves;
+  int32_t* partials = static_cast<int32_t*>(d->workspace);
+  int32_t* col_offs = partials ? partials + (int64_t)units_pad * E : nullptr;
+
+  TopkParams tp;
+  tp.logits = d->logits;
+  tp.stride_m = d->logits_stride_m;
+  tp.T = T;
+  tp.n_rows_imm = d->n_rows_ptr ? T : (d->n_rows < 0 ? T : d->n_rows);
+  tp.n_rows_ptr = d->n_rows_ptr;
+  tp.E = E;
+  tp.k = k;
+  tp.apply_softmax = d->apply_softmax;
+  tp.use_provided_indx = d->use_provided_indx;
+  tp.vals = d->vals;
+  tp.indx = static_cast<int16_t*>(d->indx);
+  tp.bitmatrix = static_cast<uint32_t*>(d->bitmatrix);
+  tp.bm_stride_w = d->bitmatrix_stride_w;
+  tp.partials = want_meta ? partials : nullptr;
+  tp.rows_per_wave = rpw;
+  tp.fill_a = want_meta ? d->col_sorted_indx : nullptr;
+  tp.fill_b = want_meta ? d->row_sorted_indx : nullptr;
+  tp.fill_c = want_meta ? d->gather_indx : nullptr;
+  int32_t rc;
+  if (d->logits_dtype == TK_F32 || !d->logits)
+    rc = launch_topk<TK_F32>(tp, units, st);
+  else if (d->logits_dtype == TK_BF16)
+    rc = launch_topk<TK_BF16>(tp, units, st);
+  else if (d->logits_dtype == TK_F16)
+    rc = launch_topk<TK_F16>(tp, units, st);
+  else
+    return fail(TK_ERR_UNSUPPORTED, "tk_route: logits dtype %d", d->logits_dtype);
+  if (rc != TK_OK || !want_meta) return rc;
+
+  RaggedOut ro;
+  ro.slice_offs = d->slice_offs;
+  ro.block_offs = d->block_offs;
+  ro.block_offs_stride = d->block_offs_stride;
+  ro.block_sched = d->block_schedule;
+  ro.block_sched_stride = d->block_schedule_stride;
+  ro.max_n_blocks = d->max_n_blocks;
+  const int want_ragged = d->slice_offs != nullptr;
+  if (want_ragged && (!d->block_offs || (!d->block_schedule && d->max_n_blocks > 0))) return fail(TK_ERR_INVALID, "tk_route: incomplete ragged outputs");
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, partials, units, E, d->col_sum, col_offs, want_ragged, ro);
+  rc = check_launch("route_scan_kernel");
+  if (rc != TK_OK) return rc;
+
+  ScatterParams sp;
+  sp.indx16 = static_cast<const int16_t*>(d->indx);
+  sp.indx32 = nullptr;
+  sp.T = T;
+  sp.k = k;
+  sp.E = E;
+  sp.n_rows_imm = tp.n_rows_imm;
+  sp.n_rows_ptr = d->n_rows_ptr;
+  sp.rows_per_wave = rpw;
+  sp.partials = partials;
+  sp.col_offs = col_offs;
+  sp.col_sorted = d->col_sorted_indx;
+  sp.row_sorted = d->row_sorted_indx;
+  sp.gather_out = d->gather_indx;
+  sp.vals = d->vals;
+  sp.gammas_out = d->vals ? d->gammas : nullptr;
+  sp.vals_bytes = (d->logits_dtype == TK_F32 || !d->logits) ? 4 : 2;
+  hipLaunchKernelGGL(route_scatter_kernel, dim3(units_pad / kWaves), dim3(kWaves * 64), 0, st, sp);
+  return check_launch("route_scatter_kernel");
+}
+
+extern "C" int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t* slice_offs, int32_t* block_offs,
+                                      int64_t block_offs_stride, int32_t* block_schedule, int64_t block_schedule_stride,
+                                      int32_t max_n_blocks, tk_stream_t stream) {
+  if (n_slices < 0 || max_n_blocks < 0) return fail(TK_ERR_INVALID, "tk_ragged_metadata: negative size");
+  if (n_slices >= 65536) return fail(TK_ERR_INVALID, "tk_ragged_metadata: at most 65535 slices");
+  if (!slice_offs || !block_offs || (!block_schedule && max_n_blocks > 0) || (!slice_sizes && n_slices > 0)) return fail(TK_ERR_INVALID, "tk_ragged_metadata: null pointer");
+  RaggedOut ro;
+  ro.slice_offs = slice_offs;
+  ro.block_offs = block_offs;
+  ro.block_offs_stride = block_offs_stride;
+  ro.block_sched = block_schedule;
+  ro.block_sched_stride = block_schedule_stride;
+  ro.max_n_blocks = max_n_blocks;
+  hipLaunchKernelGGL(ragged_metadata_kernel, dim3(1), dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), slice_sizes, n_slices, ro);
+  return check_launch("ragged_metadata_kernel");
+}

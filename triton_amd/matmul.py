@@ -1,0 +1,291 @@
+"""Ragged expert matmul host driver (mirrors `triton_kernels/matmul.py:40-142,245-766`).
+
+    Y[dst(r), :] = act((X[src(r), :] @ W[e(r)]) * scales + bias[e(r), :]) * gammas[r]
+
+Python validates, picks the tile (`opt_flags`), allocates the output with `torch.empty` and fills one
+`tk_gemm_desc`; the HIP kernel behind `tk_moe_gemm` does the rest.  Supported operand combinations:
+
+    activations  weights                        notes
+    bf16         bf16                           K-contiguous weights are used in place; N-contiguous
+                                                ones are re-laid out once per call
+    bf16         mxfp4 (uint8 e2m1 + e8m0)      dequantised in registers, bf16 MFMA, fp32 accumulate
+    fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
+
+Options of the reference signature that this build rejects with NotImplementedError: ragged-K
+(`b_ragged_metadata`), `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, MX-output epilogues, flexpoint
+scales, batched 3-D activations, split-k.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from enum import Enum, auto
+from typing import Callable
+
+import torch
+
+from . import _native as nt
+from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_opt_flags, scoped_opt_flags,  # noqa: F401
+                                        scoped_opt_flags_constraints, set_idle_sms)
+from .numerics import InFlexData, OutFlexData
+from .specialize import FnSpecs
+from .tensor import FP4, RaggedTensorMetadata, Tensor, torch_dtype_to_dtype, wrap_torch_tensor
+from .tensor_details.layout_details.strided import StridedLayout
+
+MXFP_BLOCK_SIZE = 32
+
+
+@dataclass(frozen=True)
+class FusedActivation:
+    specs: FnSpecs = FnSpecs.default()
+    fn_args: tuple = tuple()
+
+
+@dataclass(frozen=True)
+class Epilogue:
+    specs: FnSpecs = FnSpecs.default()
+    fn_arg_values_matmul: tuple = tuple()
+    fn_arg_values_finalize: tuple = tuple()
+    effective_itemsize: float | None = None
+
+
+class FnName(Enum):
+    QUANTIZE_MXFP8 = auto()
+    QUANTIZE_MXFP4 = auto()
+    QUANTIZE_NVFP4 = auto()
+
+
+@dataclass(frozen=True)
+class FusedComm:
+    """Fused all-gather / reduce-scatter store; multi-GPU only, rejected by `matmul` in this build."""
+    out_handles: torch.Tensor
+    map_dst_coord: object = None
+    all_writes_issued: object = None
+    reduce_rank: int = 0
+    n_reduce_shards: int = 1
+
+
+@dataclass(frozen=True)
+class FlexCtx:
+    lhs_data: InFlexData = InFlexData()
+    rhs_data: InFlexData = InFlexData()
+    out_data: OutFlexData = OutFlexData()
+    acc_data: InFlexData = InFlexData()
+
+
+@dataclass
+class PrecisionConfig:
+    max_num_imprecise_acc: int | None = None
+    allow_tf32: bool = True
+    flex_ctx: FlexCtx = FlexCtx()
+    acc_scale: float = 1.0
+    flexpoint_saturate_inf: bool = False
+    report_quantization_err_fn: Callable | None = None
+    a_mx_scale: torch.Tensor | Tensor | None = None
+    a_mx_tensor_scale: torch.Tensor | None = None
+    a_microblock_size: int | None = None
+    b_mx_scale: torch.Tensor | Tensor | None = None
+    b_mx_tensor_scale: torch.Tensor | None = None
+    b_microblock_size: int | None = None
+    c_mx_scale: torch.Tensor | Tensor | None = None
+    c_microblock_size: int | None = None
+    c_value_pack_factor: int = 1
+    out_dtype: torch.dtype | None = None
+    intermediate_out_dtype: torch.dtype | None = None
+    enforce_bitwise_invariance: bool = False
+
+
+def matmul_set_idle_sms(num_idle_sms):
+    set_idle_sms(num_idle_sms)
+
+
+def _flex_is_trivial(flex: FlexCtx) -> bool:
+    return (flex.lhs_data.scale is None and flex.rhs_data.scale is None and flex.acc_data.scale is None
+            and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
+            and flex.out_data.checksum_scale is None)
+
+
+def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
+    """[E, K, N] weights with unit stride along K (each output column contiguous in memory)."""
+    if w.stride(-2) == 1 and (w.shape[-2] == 1 or w.stride(-1) >= w.shape[-2]):
+        return w
+    return w.transpose(-1, -2).contiguous().transpose(-1, -2)
+
+
+def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
+           b_ragged_metadata: RaggedTensorMetadata | None = None, gather_indx: torch.Tensor | None = None,
+           scatter_indx: torch.Tensor | None = None, precision_config: PrecisionConfig | None = None,
+           betas: torch.Tensor | None = None, gammas: torch.Tensor | None = None, out_alpha: float | None = None,
+           c: torch.Tensor | None = None, fused_comm: FusedComm | None = None,
+           fused_activation: FusedActivation | None = None, epilogue: Epilogue | None = None,
+           c_acc_in: torch.Tensor | None = None):
+    """
+    Y[:, :] = 0
+    for e in experts:
+        Y[idxs_y_m(e), :] += matmul(X[idxs_x_m(e), :], W[e, :, :])
+    """
+    if b_ragged_metadata is not None:
+        raise NotImplementedError("ragged-K matmul (b_ragged_metadata) is a training feature and is not supported")
+    if c_acc_in is not None:
+        raise NotImplementedError("c_acc_in is not supported")
+    if fused_comm is not None:
+        raise NotImplementedError("fused_comm is a multi-GPU feature and is not supported")
+    if betas is not None:
+        raise NotImplementedError("betas is not supported")
+    if out_alpha is not None:
+        raise NotImplementedError("out_alpha is not supported")
+    if precision_config is None:
+        precision_config = PrecisionConfig()
+    if fused_activation is None:
+        fused_activation = FusedActivation(FnSpecs.default(), tuple())
+    if epilogue is None:
+        epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+    if epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
+        raise NotImplementedError("MX-output / custom epilogues are not supported")
+    if not _flex_is_trivial(precision_config.flex_ctx):
+        raise NotImplementedError("flexpoint scales are not supported; use a/b_mx_tensor_scale for fp8 scales")
+    if precision_config.a_mx_scale is not None:
+        raise NotImplementedError("MX-quantised activations (a_mx_scale) are not supported")
+    if isinstance(a, Tensor):
+        a = a.storage.data
+    if a.ndim != 2:
+        raise NotImplementedError("batched 3-D activations are not supported")
+    nt.require_gpu(a, "a")
+    # ---- weights -------------------------------------------------------------------------------
+    b_scale = precision_config.b_mx_scale
+    if not isinstance(b, Tensor):
+        b = wrap_torch_tensor(b, dtype=FP4 if b.dtype == torch.uint8 else None)
+    if not isinstance(b.storage.layout, StridedLayout):
+        raise NotImplementedError("only strided weight layouts are supported")
+    if b_scale is not None and not isinstance(b_scale, Tensor):
+        b_scale = wrap_torch_tensor(b_scale)
+    if b_scale is not None:
+        if not isinstance(b_scale.storage.layout, StridedLayout):
+            raise NotImplementedError("only strided MX scale layouts are supported")
+        assert b_scale.storage.data.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.storage.data.dtype}"
+        assert precision_config.b_microblock_size is None or precision_config.b_microblock_size == MXFP_BLOCK_SIZE, \
+            f"Unsupported microscale block size {precision_config.b_microblock_size}"
+    w = b.storage.data
+    if w.ndim == 2:
+        w = w[None]
+    K_W, N = b.shape[-2:]
+    M = a.shape[-2] if gather_indx is None else gather_indx.shape[0]
+    K = a.shape[-1]
+    assert K == K_W, f"reduction dims differ: a has K={K}, b has K={K_W}"
+    is_ragged = a_ragged_metadata is not None
+    n_slices = a_ragged_metadata.n_slices if is_ragged else w.shape[0]
+    if not is_ragged and w.shape[0] != 1:
+        raise NotImplementedError("batched weights need ragged metadata")
+    if is_ragged:
+        assert w.shape[0] == n_slices, f"{w.shape[0]} weight slices for {n_slices} ragged slices"
+    # ---- output --------------------------------------------------------------------------------
+    reduction_n = fused_activation.specs.reduction_n
+    act = nt.TK_ACT_NONE
+    alpha, limit, has_limit = 0.0, 0.0, 0
+    if fused_activation.specs.fn is not None or fused_activation.specs.name != "dflt":
+        if fused_activation.specs.name != "swiglu" or reduction_n != 2:
+            raise NotImplementedError(f"fused activation {fused_activation.specs.name!r} is not supported")
+        act = nt.TK_ACT_SWIGLU
+        alpha = float(fused_activation.fn_args[0])
+        lim = fused_activation.fn_args[1] if len(fused_activation.fn_args) > 1 else None
+        has_limit = int(lim is not None)
+        limit = float(lim) if lim is not None else 0.0
+    out_dtype = precision_config.out_dtype or a.dtype
+    if out_dtype != torch.bfloat16:
+        raise NotImplementedError(f"output dtype {out_dtype} is not supported (bf16 only); set precision_config.out_dtype")
+    y_rows = scatter_indx.shape[0] if scatter_indx is not None else M
+    out_shape = (y_rows, N // reduction_n)
+    if c is None:
+        c = torch.empty(out_shape, dtype=out_dtype, device=a.device)
+    else:
+        assert tuple(c.shape[-2:]) == out_shape and c.dtype == out_dtype and c.stride(-1) == 1
+        c = c.view(out_shape) if c.ndim > 2 else c
+    opt_flags = make_opt_flags(torch_dtype_to_dtype(out_dtype), torch_dtype_to_dtype(a.dtype), b.dtype, precision_config,
+                               1, M, N, K, a_ragged_metadata, epilogue_reduction_n=reduction_n)
+    if M * N == 0:
+        return c
+    if a.stride(-1) != 1:
+        a = a.contiguous()
+    d = nt.GemmDesc()
+    d.x = a.data_ptr()
+    d.x_dtype = nt.TORCH_TO_TK[a.dtype]
+    d.x_stride_m = a.stride(0)
+    a_ts = precision_config.a_mx_tensor_scale
+    if a_ts is not None:
+        a_ts = a_ts.to(torch.float32).reshape(-1).contiguous()
+        assert a_ts.numel() == a.shape[0], "a_mx_tensor_scale must hold one scale per row of a"
+        d.x_row_scale = a_ts.data_ptr()
+    keep = [a_ts]
+    if b.dtype == FP4:
+        assert b_scale is not None, "mxfp4 weights need precision_config.b_mx_scale"
+        assert w.dtype == torch.uint8
+        if w.stride(-2) != 1:
+            raise NotImplementedError("mxfp4 weights must be packed along K (stride(-2) == 1)")
+        ws = b_scale.storage.data
+        ws = ws[None] if ws.ndim == 2 else ws
+        ws = _k_contiguous(ws)
+        d.w_dtype = nt.TK_E2M1
+        d.w_mx_scale = ws.data_ptr()
+        d.ws_stride_e, d.ws_stride_k, d.ws_stride_n = ws.stride()
+        keep.append(ws)
+    else:
+        if b_scale is not None:
+            raise NotImplementedError("MX scales are supported with mxfp4 (uint8) weights only")
+        w = _k_contiguous(w)
+        d.w_dtype = nt.TORCH_TO_TK.get(w.dtype, -1)
+    d.w = w.data_ptr()
+    d.w_stride_e, d.w_stride_k, d.w_stride_n = w.stride()
+    keep.append(w)
+    b_ts = precision_config.b_mx_tensor_scale
+    if b_ts is not None:
+        b_ts = b_ts.to(torch.float32).reshape(w.shape[0], N).contiguous()
+        d.w_col_scale = b_ts.data_ptr()
+        d.wcs_stride_e = b_ts.stride(0)
+        keep.append(b_ts)
+    if bias is not None:
+        bias2 = bias[None] if bias.ndim == 1 else bias
+        if bias2.stride(-1) != 1 or bias2.dtype not in (torch.float32, torch.bfloat16):
+            bias2 = bias2.to(torch.float32).contiguous()
+        d.bias = bias2.data_ptr()
+        d.bias_dtype = nt.TORCH_TO_TK[bias2.dtype]
+        d.bias_stride_e = bias2.stride(0)
+        keep.append(bias2)
+    if gather_indx is not None:
+        assert gather_indx.dtype == torch.int32
+        gather_indx = gather_indx.contiguous()
+        d.gather_indx = gather_indx.data_ptr()
+    if scatter_indx is not None:
+        assert scatter_indx.dtype == torch.int32
+        scatter_indx = scatter_indx.contiguous()
+        d.scatter_indx = scatter_indx.data_ptr()
+        d.scatter_len = scatter_indx.shape[0]
+    if gammas is not None:
+        g = gammas if gammas.dtype in (torch.float32, torch.bfloat16) else gammas.to(torch.float32)
+        g = g.contiguous()
+        d.gammas = g.data_ptr()
+        d.gammas_dtype = nt.TORCH_TO_TK[g.dtype]
+        keep.append(g)
+    block_m = opt_flags.block_m
+    if is_ragged:
+        md = a_ragged_metadata
+        d.slice_sizes = md.slice_sizes.data_ptr()
+        d.slice_offs = md.slice_offs.data_ptr()
+        bo, bs = md.block_offs(block_m), md.block_schedule(block_m)
+        assert bo.stride(0) == 1 and (bs.numel() == 0 or bs.stride(0) == 1)
+        d.block_offs = bo.data_ptr()
+        d.block_schedule = bs.data_ptr()
+        d.n_slices = n_slices
+        d.grid_m = min(RaggedTensorMetadata.n_blocks(n_slices, M, block_m), bs.shape[0])
+    else:
+        d.n_slices = 1
+        d.grid_m = (M + block_m - 1) // block_m
+    d.block_m = block_m
+    d.M, d.N, d.K = M, N, K
+    d.y = c.data_ptr()
+    d.y_dtype = nt.TORCH_TO_TK[c.dtype]
+    d.y_stride_m = c.stride(0)
+    d.activation = act
+    d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
+    with torch.cuda.device(a.device):
+        nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
+    del keep
+    return c

@@ -170,3 +170,38 @@ def empty(shape, dtype: DataType, device, layout=None, allow_implicit_conversion
     if allow_implicit_conversion:
         ret = convert_layout(ret, layout)
     return ret
+
+
+# ---------------------------------------------------------------------------------------------------
+# routing data classes (tensor.py:159-209 of the reference)
+# ---------------------------------------------------------------------------------------------------
+from .tensor_details import bitmatrix as bitmatrix_details  # noqa: E402
+from .tensor_details import ragged_tensor as ragged_tensor_details  # noqa: E402
+from .tensor_details.bitmatrix import BitmatrixMetadata  # noqa: E402,F401
+from .tensor_details.ragged_tensor import RaggedTensorMetadata  # noqa: E402,F401
+
+make_bitmatrix_metadata = bitmatrix_details.make_bitmatrix_metadata
+make_ragged_tensor_metadata = ragged_tensor_details.make_ragged_tensor_metadata
+remap_ragged_tensor_metadata = ragged_tensor_details.remap_ragged_tensor_metadata
+
+
+@dataclass
+class RaggedTensor:
+    """A stack of 2-D slices with a common column count, stored as one (possibly padded) 2-D tensor."""
+    slice_sizes: torch.Tensor
+    data: torch.Tensor
+    metadata: RaggedTensorMetadata
+
+
+@dataclass
+class SparseMatrix:
+    """Top-k result: `vals`/`indx` [T, k] plus the bit mask of selected columns.  `mask_metadata`
+    (histogram and permutations) is computed on construction unless the producer already has it."""
+    indx: torch.Tensor
+    vals: torch.Tensor
+    mask: Tensor
+    mask_metadata: BitmatrixMetadata | None = None
+
+    def __post_init__(self):
+        if self.mask_metadata is None:
+            self.mask_metadata = make_bitmatrix_metadata(self.indx, self.mask)

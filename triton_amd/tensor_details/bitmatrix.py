@@ -1,0 +1,101 @@
+"""Expert histogram and gather/scatter permutations of a routing bitmatrix
+(mirrors `triton_kernels/tensor_details/bitmatrix.py:8-150`)."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .. import _native as nt
+
+
+@dataclass
+class BitmatrixMetadata:
+    """
+    For the bitmatrix   [0 0 1 0 1 1 0
+                         0 1 0 0 0 1 0
+                         1 1 1 0 0 0 1
+                         0 0 1 0 1 0 0]
+    col_sum         = [1 2 3 0 2 2 1]
+    col_sorted_indx = [5 | 3 6 | 0 7 9 | | 1 10 | 2 4 | 8]   nonzeros numbered row-major, grouped by column
+    row_sorted_indx = [3 6 8 | 1 9 | 0 2 4 10 | 5 7]          its inverse permutation
+    """
+    col_sum: torch.Tensor
+    col_sorted_indx: torch.Tensor
+    row_sorted_indx: torch.Tensor
+
+
+def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_indx, vals, bitmatrix_data, want_meta,
+           want_extras=False, ragged=None):
+    """Fills and submits a tk_route_desc.  Returns a dict of the tensors it allocated."""
+    dev = indx16.device
+    T = indx16.shape[0]
+    R = T * k
+    out = {}
+    d = nt.RouteDesc()
+    d.logits = nt.ptr(logits)
+    d.logits_dtype = nt.TORCH_TO_TK[logits.dtype] if logits is not None else nt.TK_F32
+    d.logits_stride_m = logits.stride(0) if logits is not None else 0
+    d.n_tokens = T
+    if isinstance(n_rows, torch.Tensor):
+        d.n_rows = -1
+        d.n_rows_ptr = n_rows.data_ptr()
+        assert n_rows.dtype == torch.int32 and n_rows.is_cuda
+    else:
+        d.n_rows = -1 if n_rows is None else int(n_rows)
+        d.n_rows_ptr = None
+    d.n_experts = n_experts
+    d.k = k
+    d.apply_softmax = int(bool(apply_softmax))
+    d.use_provided_indx = int(bool(use_provided_indx))
+    d.vals = nt.ptr(vals)
+    d.indx = indx16.data_ptr()
+    d.indx_dtype = nt.TK_I16
+    if bitmatrix_data is not None:
+        d.bitmatrix = bitmatrix_data.data_ptr()
+        d.bitmatrix_stride_w = bitmatrix_data.stride(1)
+    if want_meta:
+        col_sum = torch.empty((n_experts, ), dtype=torch.int32, device=dev)
+        combined = torch.empty((2 * R, ), dtype=torch.int32, device=dev)
+        ws = torch.empty((max(1, nt.lib().tk_route_workspace_bytes(T, n_experts)), ), dtype=torch.uint8, device=dev)
+        out.update(col_sum=col_sum, col_sorted_indx=combined[:R], row_sorted_indx=combined[R:], _ws=ws)
+        d.col_sum = col_sum.data_ptr()
+        d.col_sorted_indx = combined.data_ptr()
+        d.row_sorted_indx = combined.data_ptr() + 4 * R
+        d.workspace = ws.data_ptr()
+        if want_extras:
+            gather = torch.empty((R, ), dtype=torch.int32, device=dev)
+            d.gather_indx = gather.data_ptr()
+            out["gather_indx"] = gather
+            if vals is not None:
+                gam = torch.empty((R, ), dtype=vals.dtype, device=dev)
+                d.gammas = gam.data_ptr()
+                out["gammas"] = gam
+        if ragged is not None:
+            slice_offs, block_offs, sched, width = ragged
+            d.slice_offs = slice_offs.data_ptr()
+            d.block_offs = block_offs.data_ptr()
+            d.block_offs_stride = block_offs.stride(0)
+            d.block_schedule = sched.data_ptr() if width > 0 else None
+            d.block_schedule_stride = sched.stride(0) if width > 0 else 0
+            d.max_n_blocks = width
+    if T > 0:
+        with torch.cuda.device(dev):
+            nt.check(nt.lib().tk_route(d, nt.stream_ptr(dev)))
+    elif want_meta:
+        out["col_sum"].zero_()
+    return out
+
+
+def make_bitmatrix_metadata(nonzero_indx, bitmatrix):
+    """`nonzero_indx [T, k]` expert ids (-1 = dropped); `bitmatrix` gives the column count and row bound."""
+    assert nonzero_indx.ndim == 2
+    nt.require_gpu(nonzero_indx, "nonzero_indx")
+    n_cols = bitmatrix.shape[1]
+    n_rows = bitmatrix.shape[0]
+    indx16 = nonzero_indx if nonzero_indx.dtype == torch.int16 else nonzero_indx.to(torch.int16)
+    indx16 = indx16.contiguous()
+    r = _route(None, indx16, n_rows, n_cols, nonzero_indx.shape[1], apply_softmax=False, use_provided_indx=True,
+               vals=None, bitmatrix_data=None, want_meta=True)
+    return BitmatrixMetadata(col_sum=r["col_sum"], col_sorted_indx=r["col_sorted_indx"],
+                             row_sorted_indx=r["row_sorted_indx"])
