@@ -1,0 +1,249 @@
+"""Benchmark of the quantized MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A "step" is one forward pass of the gpt-oss-120b-shaped MXFP4 MoE FFN (BASELINE config 3: 4096 tokens,
+d_model 2880, 128 experts, top-4, W1 [128, 2880, 5760] and W2 [128, 2880, 2880] in MXFP4 with bf16 biases):
+router -> gather-GEMM (+bias, swiglu) -> scatter-GEMM (+bias, gate weight) -> top-k combine, on synthetic
+seeded inputs resident in HBM.  Prints ONE JSON line; `value` is the layer's TFLOP/s (2*R*K*N over both
+GEMMs, R = routed rows).  `roofline` covers the dominant kernel (the first expert GEMM), timed live with
+HIP events on the launch stream; `cpu_baseline` is the CPU oracle on a bounded sample of the same
+workload; `extra` carries the decode (config 4) and MX round-trip (config 2) figures.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+
+
+def make_moe_weights(E, d_model, d_ff2, seed, device, n_copies=1):
+    """MXFP4 expert weights (+ bf16 biases) of a gpt-oss-shaped FFN, quantised along K on the GPU."""
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    out = []
+    for _ in range(n_copies):
+        w1q, w1s, w2q, w2s = [], [], [], []
+        for _e in range(E):
+            w1 = (torch.randn((d_model, d_ff2), generator=g) * 0.02).to(torch.bfloat16).to(device)
+            q, s = downcast_to_mxfp(w1[None], torch.uint8, axis=1)
+            w1q.append(q)
+            w1s.append(s)
+            w2 = (torch.randn((d_ff2 // 2, d_model), generator=g) * 0.02).to(torch.bfloat16).to(device)
+            q, s = downcast_to_mxfp(w2[None], torch.uint8, axis=1)
+            w2q.append(q)
+            w2s.append(s)
+
+        def cat(parts):
+            # keep the K-contiguous layout the quantiser produces ([E, N, K/2] in memory)
+            return torch.cat([p.transpose(1, 2) for p in parts], dim=0).contiguous().transpose(1, 2)
+
+        b1 = (torch.randn((E, d_ff2), generator=g) * 0.01).to(torch.bfloat16).to(device)
+        b2 = (torch.randn((E, d_model), generator=g) * 0.01).to(torch.bfloat16).to(device)
+        out.append(dict(w1=cat(w1q), w1s=cat(w1s), w2=cat(w2q), w2s=cat(w2s), b1=b1, b2=b2))
+    return out
+
+
+class MoeLayer:
+    """The hot path composed from the drop-in API (triton_kernels names)."""
+
+    def __init__(self, weights, k, alpha=1.702, limit=7.0):
+        from triton_kernels.legacy import routing
+        from triton_kernels.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
+        from triton_kernels.reduce import reduce
+        from triton_kernels.swiglu import swiglu_fn
+        self.routing, self.matmul, self.reduce = routing, matmul, reduce
+        self.W = weights
+        self.k = k
+        self.act = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (alpha, limit))
+        self.pc1 = PrecisionConfig(b_mx_scale=weights["w1s"])
+        self.pc2 = PrecisionConfig(b_mx_scale=weights["w2s"])
+        self.marks = None  # optional list collecting (start, end) events around the first GEMM
+
+    def set_weights(self, weights):
+        from triton_kernels.matmul import PrecisionConfig
+        self.W = weights
+        self.pc1 = PrecisionConfig(b_mx_scale=weights["w1s"])
+        self.pc2 = PrecisionConfig(b_mx_scale=weights["w2s"])
+
+    def __call__(self, x, logits):
+        W, k = self.W, self.k
+        rdata, gather, scatter = self.routing(logits, k)
+        md = rdata.expt_data
+        if self.marks is not None:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+        h = self.matmul(x, W["w1"], W["b1"], md, gather_indx=rdata.token_indx, precision_config=self.pc1,
+                        fused_activation=self.act)
+        if self.marks is not None:
+            e1.record()
+            self.marks.append((e0, e1))
+        y = self.matmul(h, W["w2"], W["b2"], md, scatter_indx=scatter.dst_indx, precision_config=self.pc2,
+                        gammas=rdata.gate_scal)
+        out, _ = self.reduce(y.view(x.shape[0], k, -1), dim=1)
+        return out, rdata
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def cpu_baseline(seed=2):
+    """CPU oracle on a bounded sample of config 3: 16 of the 128 experts and 512 tokens (top-4), which
+    keeps the ~128 routed rows per expert of the full workload."""
+    from oracle import moe as omoe
+    from oracle import mxfp as omx
+    E, T, k, d, f2 = 16, 512, 4, 2880, 5760
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g)
+    w1 = (torch.randn((E, d, f2), generator=g) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn((E, f2 // 2, d), generator=g) * 0.02).to(torch.bfloat16)
+    b1 = (torch.randn((E, f2), generator=g) * 0.01).to(torch.bfloat16)
+    b2 = (torch.randn((E, d), generator=g) * 0.01).to(torch.bfloat16)
+    w1q, w1s = omx.downcast_to_mxfp(w1, torch.uint8, axis=1)
+    w2q, w2s = omx.downcast_to_mxfp(w2, torch.uint8, axis=1)
+    del w1, w2
+    torch.set_num_threads(os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    omoe.moe_layer(x, logits, k, w1q, b1, w2q, b2, w1_mx_scale=w1s, w2_mx_scale=w2s)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * T * k * d * (f2 + d)
+    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"CPU oracle (oracle/moe.py) on {E} of 128 experts x {T} tokens, top-{k}, same per-expert shapes; "
+                f"{dt:.1f} s wall")
+
+
+def bench_decode(device, steps, warmup):
+    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched."""
+    E, k, d, f2 = 128, 4, 2880, 5760
+    copies = make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)
+    per_expert = d * f2 // 2 + d * f2 // 32 + (f2 // 2) * d // 2 + (f2 // 2) * d // 32
+    res = {}
+    g = torch.Generator().manual_seed(3)
+    ebias = torch.randn((E, ), generator=g) * 1.5
+    layer = MoeLayer(copies[0], k)
+    for T in (1, 4, 16, 64):
+        x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
+        logits = (torch.randn((T, E), generator=g) + ebias).to(device)
+        _, rdata = layer(x, logits)
+        active = int((rdata.expt_hist > 0).sum())
+        it = [0]
+
+        def step():
+            layer.set_weights(copies[it[0] % len(copies)])  # rotate weight copies: no reuse from the last-level cache
+            it[0] += 1
+            layer(x, logits)
+
+        ms = time_steps(step, steps, warmup)
+        gbytes = active * per_expert / 1e9
+        res[f"T{T}"] = dict(ms=round(ms, 4), active_experts=active, weight_GB=round(gbytes, 4),
+                            GBps=round(gbytes / (ms * 1e-3), 1), frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
+    return res
+
+
+def bench_mx(device, steps, warmup):
+    """Config 2: MX quantise / dequantise of [32, 2880, 5760] bf16 along axis 1 (2.53125 B per element each way)."""
+    from triton_kernels.numerics_details.mxfp import downcast_to_mxfp, upcast_from_mxfp
+    w = (torch.randn((32, 2880, 5760), device=device) * 0.02).to(torch.bfloat16)
+    nbytes = w.numel() * 2.53125
+    ms_q = time_steps(lambda: downcast_to_mxfp(w, torch.uint8, axis=1), steps, warmup)
+    q, s = downcast_to_mxfp(w, torch.uint8, axis=1)
+    ms_d = time_steps(lambda: upcast_from_mxfp(q, s, torch.bfloat16, axis=1), steps, warmup)
+    return dict(quant_ms=round(ms_q, 4), quant_GBps=round(nbytes / ms_q / 1e6, 1), dequant_ms=round(ms_d, 4),
+                dequant_GBps=round(nbytes / ms_d / 1e6, 1), frac_hbm_quant=round(nbytes / ms_q / 1e6 / PEAK_HBM_GBPS, 4),
+                frac_hbm_dequant=round(nbytes / ms_d / 1e6 / PEAK_HBM_GBPS, 4))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
+    ap.add_argument("--no-extra", action="store_true", help="skip the decode and MX round-trip figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (expert-parallel sharding is described in DESIGN.md)",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    T, E, k, d, f2 = 4096, 128, 4, 2880, 5760
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
+    logits = torch.randn((T, E), generator=g).to(device)
+    weights = make_moe_weights(E, d, f2, seed=2, device=device)[0]
+    layer = MoeLayer(weights, k)
+
+    for _ in range(args.warmup):
+        layer(x, logits)
+    torch.cuda.synchronize()
+    layer.marks = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        layer(x, logits)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gemm1_ms = sum(a.elapsed_time(b) for a, b in layer.marks) / len(layer.marks)
+    layer.marks = None
+
+    R = T * k
+    flops1 = 2.0 * R * d * f2
+    flops = flops1 + 2.0 * R * (f2 // 2) * d
+    achieved = flops1 / (gemm1_ms * 1e-3) / 1e12
+    rec = {
+        "metric": "MoE layer TFLOP/s + HBM GB/s (% roofline), gpt-oss-120b shape, 1 MI355X",
+        "value": round(flops / (ms * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 MFMA, fp32 accumulate (mxfp4 weights dequantised in registers)",
+        "data": "synthetic",
+        "config": {"workload": "gpt-oss-120b-shaped MXFP4 MoE FFN prefill (BASELINE config 3)", "tokens": T, "d_model": d,
+                   "experts": E, "top_k": k, "w1": [E, d, f2], "w2": [E, f2 // 2, d]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "moe_gemm_kernel (gather-GEMM W1 + bias + swiglu)", "kernel_ms": round(gemm1_ms, 4)},
+    }
+    # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
+    layer_bytes = 2.19e9
+    t_roof_ms = max(flops / (PEAK_BF16_TFLOPS * 1e12), layer_bytes / (PEAK_HBM_GBPS * 1e9)) * 1e3
+    rec["layer_roofline"] = {"t_roof_ms": round(t_roof_ms, 4), "frac": round(t_roof_ms / ms, 4),
+                             "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1)}
+    if not args.no_extra:
+        rec["extra"] = {"decode_config4": bench_decode(device, max(5, args.steps), args.warmup),
+                        "mx_round_trip_config2": bench_mx(device, max(5, args.steps), args.warmup)}
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()
