@@ -4,19 +4,23 @@
 //   Y[dst(r), :] = act( (X[src(r), :] @ W[e(r)]) * sx[src(r)] * sw[e(r), :] + bias[e(r), :] ) * gamma[r]
 //
 // Mapping onto CDNA4:
-//   * one workgroup = WAVES wave64s computes a tile of BM = 16*MF rows (of ONE expert) by
-//     BN = WAVES*NF*16 output columns; each wave owns NF 16-column fragments and ALL rows;
+//   * one workgroup (WM x WN wave64s) computes BM = WM*MFW*16 rows of ONE expert by BN = WN*NFW*16
+//     output columns; the K loop runs in stages of KC = 128*KS;
 //   * the MFMA is issued "transposed": the A operand is a 16(n) x 32(k) fragment of W^T and the B
 //     operand a 32(k) x 16(m) fragment of X^T, so a lane's 4 accumulator registers are 4 CONSECUTIVE
-//     output columns of one row (swiglu's (gate, linear) column pairs are lane-local);
-//   * weights are K-contiguous per output column ([E, N, K] in memory), which is exactly the MFMA
-//     operand order: each lane streams its own column straight from global memory into registers,
-//     16 bytes (= 32 e2m1 values = one MX block = one e8m0 scale) per 128-wide K step, and
-//     dequantises with v_cvt_scalef32_pk_bf16_fp4; W never passes through LDS and is never
-//     dequantised twice;
-//   * the (gathered) activation rows are staged once per K step through LDS (double buffered,
-//     rows padded by 16 B so that ds_read_b128 of 16 rows is bank-conflict free) and shared by all
-//     waves.
+//     output columns of one row (swiglu's (gate, linear) column pairs are lane-local) and both
+//     operands want K-contiguous data, which is how activations ([rows, K]) and the reference's MX
+//     weights ([E, N, K/2] in memory) are stored;
+//   * both operands are staged through LDS, double buffered, with global loads issued one stage ahead
+//     into registers.  Loads are shaped for the texture-address unit: 16 consecutive lanes fetch 256
+//     contiguous bytes of one activation row, 4 consecutive lanes the 64 bytes one weight column
+//     contributes to a stage; LDS rows are padded by 16 B so the ds_read_b128 of 16 rows / columns is
+//     bank-conflict free.  MXFP4 stays packed in LDS (4 bits per weight) together with its e8m0 scales
+//     and is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 right before the MFMA;
+//   * the rows of a tile are dealt to the WM row-waves in interleaved 16-row fragments and fragments
+//     past the expert's last row are skipped, so a nearly empty row block costs almost no MFMA time.
+#include <type_traits>
+
 #include "common.h"
 
 namespace tk {
@@ -55,7 +59,8 @@ struct GemmParams {
   int32_t grid_n;
   float alpha, limit;
   int32_t has_limit;
-  int32_t y_vec;  // output rows allow 8-byte vector stores
+  int32_t y_vec;     // output rows allow 16-byte vector stores
+  int32_t bias_vec;  // bias rows allow 16-byte vector loads
 };
 
 __device__ inline int xcd_remap(int pid, int total) {
@@ -80,281 +85,504 @@ __device__ inline bf16x8_t dequant8(uint32_t raw, float scale) {
   return r;
 }
 
+// s * (linear + 1), s = gate * sigmoid(alpha * gate); the reciprocal is the hardware approximation (1 ulp)
 __device__ inline float swiglu_f(float gate, float lin, float alpha, float limit, int has_limit) {
   if (has_limit) {
     gate = fminf(gate, limit);
     lin = fminf(fmaxf(lin, -limit), limit);
   }
-  const float s = gate / (1.0f + __expf(-alpha * gate));
+  const float s = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * gate));
   return fmaf(s, lin, s);
 }
 
-template <int WK, int MF, int NF, int WAVES, int KS, bool SWIGLU>
-__global__ __launch_bounds__(WAVES * 64) void moe_gemm_kernel(const GemmParams p) {
-  constexpr int BM = MF * 16;
-  constexpr int BN = WAVES * NF * 16;
-  constexpr int NT = WAVES * 64;
-  constexpr int KC = 128 * KS;           // K elements per pipeline stage
-  constexpr int PITCH = KC * 2 + 16;     // LDS row pitch in bytes
-  constexpr int NCHUNK = BM * (KC / 8);  // 16-byte pieces of one X stage
-  constexpr int CH = (NCHUNK + NT - 1) / NT;
-  constexpr int WREGS = (WK == WK_MXFP4) ? 4 : 16;  // dwords of W per lane per fragment per 128 k
+// two fp32 -> packed bf16 pair (round to nearest even), low half = a
+__device__ inline uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2][BM * PITCH];
+// FM = 16: v_mfma_f32_16x16x32_bf16 (lane = row % 16, 4 k-groups of 32 per 128-wide sub-stage).
+// FM = 32: v_mfma_f32_32x32x16_bf16 (lane = row % 32, 2 k-groups of 64), the full-rate shape on gfx950.
+template <int FM>
+struct Frag;
+template <>
+struct Frag<16> {
+  typedef f32x4_t acc_t;
+  static constexpr int NACC = 4;
+  static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  // accumulator register i of lane group h holds fragment row (= output column) n_of(i, h)
+  static __device__ __forceinline__ int n_of(int i, int h) { return h * 4 + i; }
+};
+template <>
+struct Frag<32> {
+  typedef f32x16_t acc_t;
+  static constexpr int NACC = 16;
+  static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int n_of(int i, int h) { return (i >> 2) * 8 + h * 4 + (i & 3); }
+};
 
-  const int pid = xcd_remap(blockIdx.x, gridDim.x);
-  const int pid_n = pid % p.grid_n;
-  const int pid_m = pid / p.grid_n;
-  int expert, off_m, start_m, eM;
+template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS, bool SWIGLU>
+__global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams p) {
+  typedef Frag<FM> FR;
+  constexpr int NT = WM * WN * 64;
+  constexpr int BM = WM * MFW * FM;
+  constexpr int BN = WN * NFW * FM;
+  constexpr int KC = 128 * KS;  // K elements per pipeline stage
+  constexpr int NG = 64 / FM;   // k-groups of lanes
+  constexpr int KG = 128 / NG;  // k per group per 128-wide sub-stage
+  constexpr int SPS = KG / 8;   // MFMA steps per sub-stage
+  constexpr bool MX = WK == WK_MXFP4;
+  constexpr int XPITCH = KC * 2 + 16;                    // bytes per activation row in LDS
+  constexpr int WROW = MX ? KC / 2 : KC * 2;             // weight bytes per column per stage
+  constexpr int WPITCH = WROW + 16;                      // MX: the pad holds the KC/32 scale bytes
+  constexpr int XBYTES = BM * XPITCH;
+  constexpr int STAGE = XBYTES + BN * WPITCH;
+  constexpr int XPIECES = BM * (KC / 8);                 // 16-byte pieces per stage
+  constexpr int WPIECES = BN * (WROW / 16);
+  constexpr int XCH = (XPIECES + NT - 1) / NT;
+  constexpr int WCH = (WPIECES + NT - 1) / NT;
+  constexpr int SCH = MX ? (BN * KS + NT - 1) / NT : 1;  // scale dwords (4 blocks = 128 k each)
+  constexpr bool XFULL = XPIECES % NT == 0, WFULL = WPIECES % NT == 0, SFULL = (BN * KS) % NT == 0;
+  static_assert(2 * STAGE <= 160 * 1024, "LDS budget");
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  int expert, off_m, start_m, eM, pid_n;
   if (p.slice_sizes) {
-    if (pid_m >= p.block_offs[p.n_slices]) return;
-    const int sched = p.block_sched[pid_m];
+    // The grid is an upper bound; renumber only the live tiles so that every XCD gets an equal share.
+    const int live = p.block_offs[p.n_slices] * p.grid_n;
+    if ((int)blockIdx.x >= live) return;
+    const int pid = xcd_remap(blockIdx.x, live);
+    pid_n = pid % p.grid_n;
+    const int sched = p.block_sched[pid / p.grid_n];
     expert = sched & 0xFFFF;
     off_m = (sched >> 16) * BM;
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
+    const int pid = xcd_remap(blockIdx.x, gridDim.x);
+    pid_n = pid % p.grid_n;
     expert = 0;
-    off_m = pid_m * BM;
+    off_m = (pid / p.grid_n) * BM;
     start_m = 0;
     eM = p.M;
   }
+  const int rows = (eM - off_m) < BM ? (eM - off_m) : BM;  // valid rows of this tile (>= 1)
+  const int nfrag_m = (rows + FM - 1) / FM;                // row fragments that hold valid rows
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int l16 = lane & 15, g = lane >> 4;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int mw = wave % WM, nw = wave / WM;
+  const int lr = lane % FM, h = lane / FM;
   const int K = p.K, N = p.N;
-
-  // ---- activation staging: this thread's 16-byte pieces ------------------------------------
-  const uint16_t* xptr[CH];
-  int xk[CH];      // k offset of the piece inside a stage
-  int xlds[CH];    // byte offset of the piece inside an LDS stage
-  bool xok[CH];
+  // fragment j of this wave covers tile rows (j*WM + mw)*FM .. +FM; fragments past the last valid row are skipped
+  int jcount = 0;
 #pragma unroll
-  for (int j = 0; j < CH; ++j) {
+  for (int j = 0; j < MFW; ++j) jcount += ((j * WM + mw) < nfrag_m) ? 1 : 0;
+
+  // ---- global -> register staging: this thread's 16-byte pieces -----------------------------
+  const uint16_t* xptr[XCH];
+  int xk[XCH], xlds[XCH];
+  bool xok[XCH];
+#pragma unroll
+  for (int j = 0; j < XCH; ++j) {
     const int id = tid + NT * j;
-    xok[j] = id < NCHUNK;
-    const int r = id / (KC / 8), c = id % (KC / 8);
+    const int r = (id / (KC / 8)) % BM, c = id % (KC / 8);
+    xok[j] = (XFULL || id < XPIECES) && r < nfrag_m * FM;  // fragments without valid rows are never read
     int row = off_m + r;
     row = row < eM ? row : eM - 1;
     const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
     xptr[j] = p.x + src * p.x_stride_m + c * 8;
     xk[j] = c * 8;
-    xlds[j] = r * PITCH + c * 16;
+    xlds[j] = r * XPITCH + c * 16;
   }
-  // ---- weight streaming: this lane's columns -------------------------------------------------
-  const int n_base = pid_n * BN + wave * (NF * 16);
-  const uint8_t* wptr[NF];
-  const uint8_t* sptr[NF];
-  bool nok[NF];
+  const uint8_t* wptr[WCH];
+  int wk[WCH], wlds[WCH];
+  bool wok[WCH];
+  const int n_tile = pid_n * BN;
 #pragma unroll
-  for (int f = 0; f < NF; ++f) {
-    const int n = n_base + f * 16 + l16;
-    nok[f] = n < N;
-    const int nn = nok[f] ? n : 0;
-    if (WK == WK_MXFP4) {
-      wptr[f] = p.w + expert * p.w_stride_e + nn * p.w_stride_n + g * 16;
-      sptr[f] = p.w_scale + expert * p.ws_stride_e + nn * p.ws_stride_n + g;
-    } else {
-      wptr[f] = p.w + expert * p.w_stride_e + nn * p.w_stride_n + g * 64;
-      sptr[f] = nullptr;
+  for (int j = 0; j < WCH; ++j) {
+    const int id = tid + NT * j;
+    wok[j] = WFULL || id < WPIECES;
+    const int col = (id / (WROW / 16)) % BN, part = id % (WROW / 16);
+    int n = n_tile + col;
+    n = n < N ? n : N - 1;  // columns past N are computed from a valid column and dropped in the epilogue
+    wptr[j] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)n * p.w_stride_n + part * 16;
+    wk[j] = MX ? part * 32 : part * 8;
+    wlds[j] = XBYTES + col * WPITCH + part * 16;
+  }
+  const uint8_t* sptr[SCH];
+  int sk[SCH], slds[SCH];
+  bool sok[SCH];
+  if constexpr (MX) {
+#pragma unroll
+    for (int j = 0; j < SCH; ++j) {
+      const int id = tid + NT * j;
+      sok[j] = SFULL || id < BN * KS;
+      const int col = (id / KS) % BN, part = id % KS;
+      int n = n_tile + col;
+      n = n < N ? n : N - 1;
+      sptr[j] = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)n * p.ws_stride_n + part * 4;
+      sk[j] = part * 128;
+      slds[j] = XBYTES + col * WPITCH + WROW + part * 4;
     }
   }
 
-  f32x4_t acc[NF][MF];
+  typename FR::acc_t acc[NFW][MFW];
 #pragma unroll
-  for (int f = 0; f < NF; ++f)
+  for (int f = 0; f < NFW; ++f)
 #pragma unroll
-    for (int m = 0; m < MF; ++m) acc[f][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < MFW; ++j)
+#pragma unroll
+      for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
 
-  uint4 xreg[CH];
-  uint32_t wreg[2][KS][NF][WREGS];
-  uint32_t sreg[2][KS][NF];
+  uint4 xreg[XCH];
+  uint4 wreg[WCH];
+  uint32_t sreg[SCH];
 
-  auto load_x = [&](int kc) {
+  // TAIL = the stage may reach past K: pieces beyond K are zero-filled (zero weights x finite activations)
+  auto load_stage = [&](auto tail_c, int kc) __attribute__((always_inline)) {
+    constexpr bool TAIL = decltype(tail_c)::value;
 #pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      if (xok[j] && kc + xk[j] < K)
+    for (int j = 0; j < XCH; ++j) {
+      if (xok[j] && (!TAIL || kc + xk[j] < K))
         xreg[j] = *reinterpret_cast<const uint4*>(xptr[j] + kc);
       else
         xreg[j] = make_uint4(0, 0, 0, 0);
     }
-  };
-  auto store_x = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < CH; ++j)
-      if (xok[j]) *reinterpret_cast<uint4*>(&lds[buf][xlds[j]]) = xreg[j];
-  };
-  auto load_w = [&](int slot, int kc) {
+    for (int j = 0; j < WCH; ++j) {
+      if ((WFULL || wok[j]) && (!TAIL || kc + wk[j] < K))
+        wreg[j] = *reinterpret_cast<const uint4*>(wptr[j] + (MX ? kc / 2 : kc * 2));
+      else
+        wreg[j] = make_uint4(0, 0, 0, 0);
+    }
+    if constexpr (MX) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int k0 = kc + s * 128 + g * 32;  // first k this lane holds in the sub-step
-#pragma unroll
-      for (int f = 0; f < NF; ++f) {
-        if constexpr (WK == WK_MXFP4) {
-          if (nok[f] && k0 < K) {
-            const uint4 v = *reinterpret_cast<const uint4*>(wptr[f] + (kc + s * 128) / 2);
-            wreg[slot][s][f][0] = v.x;
-            wreg[slot][s][f][1] = v.y;
-            wreg[slot][s][f][2] = v.z;
-            wreg[slot][s][f][3] = v.w;
-            sreg[slot][s][f] = sptr[f][(kc + s * 128) / 32];
-          } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) wreg[slot][s][f][i] = 0;
-            sreg[slot][s][f] = 127;
-          }
+      for (int j = 0; j < SCH; ++j) {
+        if (!(SFULL || sok[j])) {
+          sreg[j] = 0x7F7F7F7Fu;
+        } else if (!TAIL) {
+          uint32_t v;
+          __builtin_memcpy(&v, sptr[j] + kc / 32, 4);  // 4 consecutive e8m0 bytes, any alignment
+          sreg[j] = v;
         } else {
+          uint32_t v = 0;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (nok[f] && k0 + 8 * i < K) {
-              const uint4 v = *reinterpret_cast<const uint4*>(wptr[f] + (kc + s * 128) * 2 + i * 16);
-              wreg[slot][s][f][4 * i + 0] = v.x;
-              wreg[slot][s][f][4 * i + 1] = v.y;
-              wreg[slot][s][f][4 * i + 2] = v.z;
-              wreg[slot][s][f][4 * i + 3] = v.w;
-            } else {
-#pragma unroll
-              for (int q = 0; q < 4; ++q) wreg[slot][s][f][4 * i + q] = 0;
-            }
+          for (int b = 0; b < 4; ++b) {
+            const int k0 = kc + sk[j] + 32 * b;
+            const uint32_t byte = k0 < K ? (uint32_t)sptr[j][kc / 32 + b] : 127u;
+            v |= byte << (8 * b);
           }
+          sreg[j] = v;
         }
       }
     }
   };
-  auto compute = [&](int buf, int slot) {
+  auto store_stage = [&](int buf) __attribute__((always_inline)) {
+    uint8_t* base = lds + buf * STAGE;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      float scl[NF];
-      if constexpr (WK == WK_MXFP4) {
+    for (int j = 0; j < XCH; ++j)
+      if (xok[j]) *reinterpret_cast<uint4*>(base + xlds[j]) = xreg[j];
 #pragma unroll
-        for (int f = 0; f < NF; ++f) scl[f] = bits_f32(sreg[slot][s][f] << 23);
+    for (int j = 0; j < WCH; ++j)
+      if (WFULL || wok[j]) *reinterpret_cast<uint4*>(base + wlds[j]) = wreg[j];
+    if constexpr (MX) {
+#pragma unroll
+      for (int j = 0; j < SCH; ++j)
+        if (SFULL || sok[j]) *reinterpret_cast<uint32_t*>(base + slds[j]) = sreg[j];
+    }
+  };
+  // MFMA step t of a stage: sub-stage s = t / SPS, i = t % SPS; lane group h supplies k = s*128 + h*KG + i*8 .. +8
+  auto read_xf = [&](const uint8_t* base, int t, bf16x8_t (&xf)[MFW]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j)
+      xf[j] = *reinterpret_cast<const bf16x8_t*>(base + ((j * WM + mw) * FM + lr) * XPITCH +
+                                                  ((t / SPS) * 128 + h * KG + (t % SPS) * 8) * 2);
+  };
+  // FULL: every row fragment of this wave holds valid rows; the body is then one straight-line block in
+  // which the scheduler is told to alternate MFMAs with the dequantisation / LDS reads of the next step.
+  auto compute = [&](auto full_c, int buf) __attribute__((always_inline)) {
+    constexpr bool FULL = decltype(full_c)::value;
+    const uint8_t* base = lds + buf * STAGE;
+    const uint8_t* wbase = base + XBYTES + (nw * NFW * FM + lr) * WPITCH;
+    constexpr int STEPS = KS * SPS;
+    bf16x8_t xf[2][MFW];
+    bf16x8_t wf[2][NFW];
+    uint32_t wraw[NFW][KG / 8];  // KG e2m1 values of this lane's column (current sub-stage)
+    uint32_t sd[NFW];            // the sub-stage's 4 scale bytes of this lane's column
+    auto read_w = [&](int sub) __attribute__((always_inline)) {
+      if constexpr (MX) {
+#pragma unroll
+        for (int f = 0; f < NFW; ++f) {
+#pragma unroll
+          for (int q = 0; q < KG / 32; ++q) {
+            const uint4 v = *reinterpret_cast<const uint4*>(wbase + f * FM * WPITCH + sub * 64 + h * (KG / 2) + q * 16);
+            wraw[f][4 * q + 0] = v.x;
+            wraw[f][4 * q + 1] = v.y;
+            wraw[f][4 * q + 2] = v.z;
+            wraw[f][4 * q + 3] = v.w;
+          }
+          sd[f] = *reinterpret_cast<const uint32_t*>(wbase + f * FM * WPITCH + WROW + sub * 4);
+        }
+      }
+    };
+    auto make_wf = [&](int t, bf16x8_t (&out)[NFW]) __attribute__((always_inline)) {
+      const int sub = t / SPS, i = t % SPS;
+#pragma unroll
+      for (int f = 0; f < NFW; ++f) {
+        if constexpr (MX) {
+          const int blk = h * (KG / 32) + i / 4;  // MX block (of the sub-stage's 4) this step's 8 values lie in
+          out[f] = dequant8(wraw[f][i], bits_f32(((sd[f] >> (8 * blk)) & 0xFFu) << 23));
+        } else {
+          out[f] = *reinterpret_cast<const bf16x8_t*>(wbase + f * FM * WPITCH + (sub * 128 + h * KG + i * 8) * 2);
+        }
+      }
+    };
+    read_w(0);
+    read_xf(base, 0, xf[0]);
+    make_wf(0, wf[0]);
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const int cur = t & 1, nxt = cur ^ 1;
+      if (t + 1 < STEPS) {
+        if ((t + 1) % SPS == 0) read_w((t + 1) / SPS);
+        read_xf(base, t + 1, xf[nxt]);
+        make_wf(t + 1, wf[nxt]);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        bf16x8_t xf[MF];
+      for (int j = 0; j < MFW; ++j) {
+        if (FULL || j < jcount) {
 #pragma unroll
-        for (int m = 0; m < MF; ++m)
-          xf[m] = *reinterpret_cast<const bf16x8_t*>(&lds[buf][(m * 16 + l16) * PITCH + (s * 128 + g * 32 + i * 8) * 2]);
+          for (int f = 0; f < NFW; ++f) acc[f][j] = FR::mma(wf[cur][f], xf[cur][j], acc[f][j]);
+        }
+      }
+      if constexpr (FULL) {
+        // per MFMA: the share of the next step's VALU work (4 conversions per weight fragment) and LDS reads
+        constexpr int NM = MFW * NFW;
+        constexpr int VPM = MX ? (4 * NFW + NM - 1) / NM + 1 : 0;
 #pragma unroll
-        for (int f = 0; f < NF; ++f) {
-          bf16x8_t wf;
-          if constexpr (WK == WK_MXFP4) {
-            wf = dequant8(wreg[slot][s][f][i], scl[f]);
-          } else {
-            uint4 raw = make_uint4(wreg[slot][s][f][4 * i + 0], wreg[slot][s][f][4 * i + 1],
-                                   wreg[slot][s][f][4 * i + 2], wreg[slot][s][f][4 * i + 3]);
-            wf = __builtin_bit_cast(bf16x8_t, raw);
-          }
-#pragma unroll
-          for (int m = 0; m < MF; ++m) acc[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[m], acc[f][m], 0, 0, 0);
+        for (int m = 0; m < NM; ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (m < MFW + (MX ? 0 : NFW)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (VPM) __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
         }
       }
     }
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  auto compute_any = [&](int buf) __attribute__((always_inline)) {
+    if (jcount == MFW)
+      compute(T_{}, buf);
+    else
+      compute(F_{}, buf);
   };
 
+  // Pipeline: registers hold stage c+1 (loaded while stage c-1 was computed); at the top of stage c they go
+  // to the other LDS buffer, the loads of stage c+2 are issued, then stage c is computed from LDS.
   const int nstages = (K + KC - 1) / KC;
-  load_x(0);
-  load_w(0, 0);
-  store_x(0);
+  const int nfull = K / KC;  // stages that lie entirely below K
+  auto load_any = [&](int cs) __attribute__((always_inline)) {
+    if (cs < nfull)
+      load_stage(F_{}, cs * KC);
+    else
+      load_stage(T_{}, cs * KC);
+  };
+  load_any(0);
+  store_stage(0);
+  if (nstages > 1) load_any(1);
   __syncthreads();
   for (int c = 0; c < nstages; ++c) {
-    const int cur = c & 1;
-    const bool more = c + 1 < nstages;
-    if (more) {
-      load_x((c + 1) * KC);
-      load_w(cur ^ 1, (c + 1) * KC);
-    }
-    compute(cur, cur);
-    if (more) store_x(cur ^ 1);
+    if (c + 1 < nstages) store_stage((c + 1) & 1);
+    if (c + 2 < nstages) load_any(c + 2);
+    compute_any(c & 1);
     __syncthreads();
   }
 
   // ---- epilogue ------------------------------------------------------------------------------
+  // order: row/column scales, bias, activation, gate weight, (scattered) store
   const int NOUT = SWIGLU ? N / 2 : N;
+  const bool full_n = n_tile + BN <= N;
+  if (p.x_row_scale || p.w_col_scale) {  // fp8-style per-row x per-column scales (rare path)
 #pragma unroll
-  for (int m = 0; m < MF; ++m) {
-    const int row = off_m + m * 16 + l16;  // row inside the slice
-    if (row >= eM) continue;
-    const int srow = start_m + row;  // row in expert-sorted order
-    float rs = 1.0f;
-    if (p.x_row_scale) rs = p.x_row_scale[p.gather ? p.gather[srow] : srow];
-    float gam = 1.0f;
-    if (p.gammas) gam = load_scalar(p.gammas, srow, p.gammas_is_f32);
-    int64_t dst = srow;
-    if (p.scatter) {
-      dst = srow < p.scatter_len ? p.scatter[srow] : -1;
-      if (dst < 0) continue;
+    for (int j = 0; j < MFW; ++j) {
+      const int row = off_m + (j * WM + mw) * FM + lr;
+      float rs = 1.0f;
+      if (p.x_row_scale && row < eM) rs = p.x_row_scale[p.gather ? p.gather[start_m + row] : start_m + row];
+#pragma unroll
+      for (int f = 0; f < NFW; ++f)
+#pragma unroll
+        for (int i = 0; i < FR::NACC; ++i) {
+          const int n = n_tile + (nw * NFW + f) * FM + FR::n_of(i, h);
+          float cs = 1.0f;
+          if (p.w_col_scale && n < N) cs = p.w_col_scale[expert * p.wcs_stride_e + n];
+          acc[f][j][i] *= rs * cs;
+        }
     }
-    uint16_t* yrow = p.y + dst * p.y_stride_m;
+  }
+  if (p.bias) {
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      const int n0 = n_base + f * 16 + g * 4;
-      float v[4];
+    for (int f = 0; f < NFW; ++f)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + i;
-        float a = acc[f][m][i];
-        if (n < N) {
-          if (p.w_col_scale) a *= rs * p.w_col_scale[expert * p.wcs_stride_e + n];
-          else a *= rs;
-          if (p.bias) a += load_scalar(p.bias, expert * p.bias_stride_e + n, p.bias_is_f32);
+      for (int q = 0; q < FR::NACC / 4; ++q) {
+        const int n0 = n_tile + (nw * NFW + f) * FM + FR::n_of(4 * q, h);  // 4 consecutive columns
+        float b4[4];
+        const int64_t bo = expert * p.bias_stride_e + n0;
+        if (full_n && p.bias_vec) {
+          if (p.bias_is_f32) {
+            const float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(p.bias) + bo);
+            b4[0] = t.x, b4[1] = t.y, b4[2] = t.z, b4[3] = t.w;
+          } else {
+            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p.bias) + bo);
+            b4[0] = bits_f32(t.x << 16), b4[1] = bits_f32(t.x & 0xFFFF0000u);
+            b4[2] = bits_f32(t.y << 16), b4[3] = bits_f32(t.y & 0xFFFF0000u);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) b4[i] = n0 + i < N ? load_scalar(p.bias, bo + i, p.bias_is_f32) : 0.f;
         }
-        v[i] = a;
+#pragma unroll
+        for (int j = 0; j < MFW; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] += b4[i];
       }
-      if (SWIGLU) {
-        const int o0 = n0 / 2;
-        const float r0 = swiglu_f(v[0], v[1], p.alpha, p.limit, p.has_limit) * gam;
-        const float r1 = swiglu_f(v[2], v[3], p.alpha, p.limit, p.has_limit) * gam;
-        if (o0 + 1 < NOUT && p.y_vec) {
-          *reinterpret_cast<uint32_t*>(yrow + o0) = (uint32_t)f32_to_bf16_bits(r0) | ((uint32_t)f32_to_bf16_bits(r1) << 16);
-        } else {
-          if (o0 < NOUT) yrow[o0] = f32_to_bf16_bits(r0);
-          if (o0 + 1 < NOUT) yrow[o0 + 1] = f32_to_bf16_bits(r1);
-        }
-      } else {
-        if (n0 + 3 < N && p.y_vec) {
-          const uint32_t lo = (uint32_t)f32_to_bf16_bits(v[0] * gam) | ((uint32_t)f32_to_bf16_bits(v[1] * gam) << 16);
-          const uint32_t hi = (uint32_t)f32_to_bf16_bits(v[2] * gam) | ((uint32_t)f32_to_bf16_bits(v[3] * gam) << 16);
-          *reinterpret_cast<uint2*>(yrow + n0) = make_uint2(lo, hi);
+  }
+  // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
+  // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
+  constexpr int VW = FM == 32 ? 8 : 4;
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const int row = off_m + (j * WM + mw) * FM + lr;  // row inside the slice
+    const int srow = start_m + row;                   // row in expert-sorted order
+    bool ok = row < eM;
+    float gam = 1.0f;
+    int64_t dst = srow;
+    if (ok) {
+      if (p.gammas) gam = load_scalar(p.gammas, srow, p.gammas_is_f32);
+      if (p.scatter) {
+        dst = srow < p.scatter_len ? p.scatter[srow] : -1;
+        ok = dst >= 0;
+      }
+    }
+    uint16_t* yrow = p.y + (ok ? dst : 0) * p.y_stride_m;
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) {
+#pragma unroll
+      for (int u = 0; u < FR::NACC / VW; ++u) {
+        float v[VW];
+        int n0;
+        if constexpr (FM == 32) {
+          // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint32_t lo = f32_bits(acc[f][j][8 * u + i]), hi = f32_bits(acc[f][j][8 * u + 4 + i]);
+            auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo's upper half <-> hi's lower half
+            v[i] = bits_f32(r[0]);
+            v[4 + i] = bits_f32(r[1]);
+          }
+          n0 = n_tile + (nw * NFW + f) * FM + 16 * u + 8 * h;
         } else {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (n0 + i < N) yrow[n0 + i] = f32_to_bf16_bits(v[i] * gam);
+          for (int i = 0; i < 4; ++i) v[i] = acc[f][j][4 * u + i];
+          n0 = n_tile + (nw * NFW + f) * FM + FR::n_of(4 * u, h);
+        }
+        if (!ok) continue;
+        if (SWIGLU) {
+          float r[VW / 2];
+#pragma unroll
+          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[2 * i], v[2 * i + 1], p.alpha, p.limit, p.has_limit) * gam;
+          const int o0 = n0 / 2;
+          if (o0 + VW / 2 <= NOUT && p.y_vec) {
+            uint32_t w[VW / 4];
+#pragma unroll
+            for (int i = 0; i < VW / 4; ++i) w[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint2*>(yrow + o0) = make_uint2(w[0], w[VW / 4 - 1]);
+            else
+              *reinterpret_cast<uint32_t*>(yrow + o0) = w[0];
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i)
+              if (o0 + i < NOUT) yrow[o0 + i] = f32_to_bf16_bits(r[i]);
+          }
+        } else {
+          if (n0 + VW <= N && p.y_vec) {
+            uint32_t w[VW / 2];
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[2 * i] * gam, v[2 * i + 1] * gam);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint4*>(yrow + n0) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
+            else
+              *reinterpret_cast<uint2*>(yrow + n0) = make_uint2(w[0], w[1]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW; ++i)
+              if (n0 + i < N) yrow[n0 + i] = f32_to_bf16_bits(v[i] * gam);
+          }
         }
       }
     }
   }
 }
 
-template <int WK, int MF, int NF, int WAVES, int KS>
+template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
 int32_t launch_cfg(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
-  constexpr int BN = WAVES * NF * 16;
+  constexpr int BM = WM * MFW * FM;
+  constexpr int BN = WN * NFW * FM;
+  constexpr int KC = 128 * KS;
+  constexpr int WROW = WK == WK_MXFP4 ? KC / 2 : KC * 2;
+  constexpr int LDS_BYTES = 2 * (BM * (KC * 2 + 16) + BN * (WROW + 16));
   GemmParams q = p;
   q.grid_n = (int)cdiv(p.N, BN);
   const int64_t grid = (int64_t)grid_m * q.grid_n;
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
-  if (swiglu)
-    hipLaunchKernelGGL((moe_gemm_kernel<WK, MF, NF, WAVES, KS, true>), dim3((unsigned)grid), dim3(WAVES * 64), 0, st, q);
-  else
-    hipLaunchKernelGGL((moe_gemm_kernel<WK, MF, NF, WAVES, KS, false>), dim3((unsigned)grid), dim3(WAVES * 64), 0, st, q);
-  return check_launch("moe_gemm_kernel");
+  auto launch = [&](auto kern) -> int32_t {
+    static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
+    if (!attr_done && LDS_BYTES > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
+      attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), LDS_BYTES, st, q);
+    return check_launch("moe_gemm_kernel");
+  };
+  if (swiglu) return launch(moe_gemm_kernel<WK, FM, WM, WN, MFW, NFW, KS, true>);
+  return launch(moe_gemm_kernel<WK, FM, WM, WN, MFW, NFW, KS, false>);
 }
 
 template <int WK>
 int32_t launch_wk(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st) {
-  switch (block_m) {
-    case 16:
-      return launch_cfg<WK, 1, 2, 4, 2>(p, grid_m, swiglu, st);
-    case 32:
-      return launch_cfg<WK, 2, 2, 4, 2>(p, grid_m, swiglu, st);
-    case 64:
-      return launch_cfg<WK, 4, 4, 4, 1>(p, grid_m, swiglu, st);
-    case 128:
-      return launch_cfg<WK, 8, 4, 4, 1>(p, grid_m, swiglu, st);
-    default:
-      return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64 or 128 (got %d)", block_m);
+  //                      FM  WM WN MFW NFW KS
+  if constexpr (WK == WK_MXFP4) {
+    switch (block_m) {
+      case 16:
+        return launch_cfg<WK, 16, 1, 4, 1, 2, 2>(p, grid_m, swiglu, st);
+      case 32:
+        return launch_cfg<WK, 16, 1, 4, 2, 2, 2>(p, grid_m, swiglu, st);
+      case 64:
+        return launch_cfg<WK, 32, 2, 2, 1, 4, 1>(p, grid_m, swiglu, st);
+      case 128:
+        return launch_cfg<WK, 32, 2, 2, 2, 4, 1>(p, grid_m, swiglu, st);
+    }
+  } else {
+    switch (block_m) {
+      case 16:
+        return launch_cfg<WK, 16, 1, 4, 1, 2, 1>(p, grid_m, swiglu, st);
+      case 32:
+        return launch_cfg<WK, 16, 1, 4, 2, 2, 1>(p, grid_m, swiglu, st);
+      case 64:
+        return launch_cfg<WK, 32, 2, 2, 1, 2, 1>(p, grid_m, swiglu, st);
+      case 128:
+        return launch_cfg<WK, 32, 2, 2, 2, 2, 1>(p, grid_m, swiglu, st);
+    }
   }
+  return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64 or 128 (got %d)", block_m);
 }
 
 }  // namespace
@@ -409,7 +637,8 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.alpha = d->act_alpha;
   p.limit = d->act_limit;
   p.has_limit = d->act_has_limit;
-  p.y_vec = (d->y_stride_m % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->y) & 7) == 0);
+  p.y_vec = (d->y_stride_m % 8 == 0) && ((reinterpret_cast<uintptr_t>(d->y) & 15) == 0);
+  p.bias_vec = d->bias && (d->bias_stride_e % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->bias) & 15) == 0);
   p.grid_n = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
