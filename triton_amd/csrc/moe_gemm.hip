@@ -26,10 +26,11 @@
 namespace tk {
 namespace {
 
-enum { WK_BF16 = 0, WK_MXFP4 = 1 };
+enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3
 
 struct GemmParams {
-  const uint16_t* x;
+  const uint8_t* x;    // bf16 or e4m3 rows
+  int32_t x_is_fp8;
   int64_t x_stride_m;
   const float* x_row_scale;
   const uint8_t* w;
@@ -136,12 +137,14 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
   constexpr int KG = 128 / NG;  // k per group per 128-wide sub-stage
   constexpr int SPS = KG / 8;   // MFMA steps per sub-stage
   constexpr bool MX = WK == WK_MXFP4;
+  constexpr bool F8 = WK == WK_FP8;  // e4m3 weights AND e4m3 activations, both expanded to bf16 for the MFMA
+  constexpr int XE = F8 ? 16 : 8;    // activation elements per 16-byte global piece
   constexpr int XPITCH = KC * 2 + 16;                    // bytes per activation row in LDS
-  constexpr int WROW = MX ? KC / 2 : KC * 2;             // weight bytes per column per stage
+  constexpr int WROW = MX ? KC / 2 : (F8 ? KC : KC * 2);  // weight bytes per column per stage
   constexpr int WPITCH = WROW + 16;                      // MX: the pad holds the KC/32 scale bytes
   constexpr int XBYTES = BM * XPITCH;
   constexpr int STAGE = XBYTES + BN * WPITCH;
-  constexpr int XPIECES = BM * (KC / 8);                 // 16-byte pieces per stage
+  constexpr int XPIECES = BM * (KC / XE);                // 16-byte global pieces per stage
   constexpr int WPIECES = BN * (WROW / 16);
   constexpr int XCH = (XPIECES + NT - 1) / NT;
   constexpr int WCH = (WPIECES + NT - 1) / NT;
@@ -185,20 +188,20 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
   for (int j = 0; j < MFW; ++j) jcount += ((j * WM + mw) < nfrag_m) ? 1 : 0;
 
   // ---- global -> register staging: this thread's 16-byte pieces -----------------------------
-  const uint16_t* xptr[XCH];
+  const uint8_t* xptr[XCH];
   int xk[XCH], xlds[XCH];
   bool xok[XCH];
 #pragma unroll
   for (int j = 0; j < XCH; ++j) {
     const int id = tid + NT * j;
-    const int r = (id / (KC / 8)) % BM, c = id % (KC / 8);
+    const int r = (id / (KC / XE)) % BM, c = id % (KC / XE);
     xok[j] = (XFULL || id < XPIECES) && r < nfrag_m * FM;  // fragments without valid rows are never read
     int row = off_m + r;
     row = row < eM ? row : eM - 1;
     const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
-    xptr[j] = p.x + src * p.x_stride_m + c * 8;
-    xk[j] = c * 8;
-    xlds[j] = r * XPITCH + c * 16;
+    xptr[j] = p.x + (src * p.x_stride_m + c * XE) * (F8 ? 1 : 2);
+    xk[j] = c * XE;
+    xlds[j] = r * XPITCH + c * XE * 2;
   }
   const uint8_t* wptr[WCH];
   int wk[WCH], wlds[WCH];
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
     int n = n_tile + col;
     n = n < N ? n : N - 1;  // columns past N are computed from a valid column and dropped in the epilogue
     wptr[j] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)n * p.w_stride_n + part * 16;
-    wk[j] = MX ? part * 32 : part * 8;
+    wk[j] = MX ? part * 32 : (F8 ? part * 16 : part * 8);
     wlds[j] = XBYTES + col * WPITCH + part * 16;
   }
   const uint8_t* sptr[SCH];
@@ -250,14 +253,14 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 #pragma unroll
     for (int j = 0; j < XCH; ++j) {
       if (xok[j] && (!TAIL || kc + xk[j] < K))
-        xreg[j] = *reinterpret_cast<const uint4*>(xptr[j] + kc);
+        xreg[j] = *reinterpret_cast<const uint4*>(xptr[j] + kc * (F8 ? 1 : 2));
       else
         xreg[j] = make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int j = 0; j < WCH; ++j) {
       if ((WFULL || wok[j]) && (!TAIL || kc + wk[j] < K))
-        wreg[j] = *reinterpret_cast<const uint4*>(wptr[j] + (MX ? kc / 2 : kc * 2));
+        wreg[j] = *reinterpret_cast<const uint4*>(wptr[j] + (MX ? kc / 2 : (F8 ? kc : kc * 2)));
       else
         wreg[j] = make_uint4(0, 0, 0, 0);
     }
@@ -287,7 +290,21 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
     uint8_t* base = lds + buf * STAGE;
 #pragma unroll
     for (int j = 0; j < XCH; ++j)
-      if (xok[j]) *reinterpret_cast<uint4*>(base + xlds[j]) = xreg[j];
+      if (xok[j]) {
+        if constexpr (F8) {  // 16 e4m3 -> 16 bf16 (exact)
+          const uint32_t w4[4] = {xreg[j].x, xreg[j].y, xreg[j].z, xreg[j].w};
+          uint32_t o[8];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            o[2 * q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w4[q], 1.0f, false));
+            o[2 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w4[q], 1.0f, true));
+          }
+          *reinterpret_cast<uint4*>(base + xlds[j]) = make_uint4(o[0], o[1], o[2], o[3]);
+          *reinterpret_cast<uint4*>(base + xlds[j] + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+        } else {
+          *reinterpret_cast<uint4*>(base + xlds[j]) = xreg[j];
+        }
+      }
 #pragma unroll
     for (int j = 0; j < WCH; ++j)
       if (WFULL || wok[j]) *reinterpret_cast<uint4*>(base + wlds[j]) = wreg[j];
@@ -339,7 +356,16 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
           const int blk = h * (KG / 32) + i / 4;  // MX block (of the sub-stage's 4) this step's 8 values lie in
           out[f] = dequant8(wraw[f][i], bits_f32(((sd[f] >> (8 * blk)) & 0xFFu) << 23));
         } else {
-          out[f] = *reinterpret_cast<const bf16x8_t*>(wbase + f * FM * WPITCH + (sub * 128 + h * KG + i * 8) * 2);
+          if constexpr (F8) {  // 8 e4m3 -> 8 bf16 (exact)
+            const uint2 raw = *reinterpret_cast<const uint2*>(wbase + f * FM * WPITCH + sub * 128 + h * KG + i * 8);
+            const bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false);
+            const bf16x2_t b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
+            const bf16x2_t c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.y, 1.0f, false);
+            const bf16x2_t d2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.y, 1.0f, true);
+            out[f] = bf16x8_t{a[0], a[1], b[0], b[1], c2[0], c2[1], d2[0], d2[1]};
+          } else {
+            out[f] = *reinterpret_cast<const bf16x8_t*>(wbase + f * FM * WPITCH + (sub * 128 + h * KG + i * 8) * 2);
+          }
         }
       }
     };
@@ -535,7 +561,7 @@ int32_t launch_cfg(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   constexpr int BM = WM * MFW * FM;
   constexpr int BN = WN * NFW * FM;
   constexpr int KC = 128 * KS;
-  constexpr int WROW = WK == WK_MXFP4 ? KC / 2 : KC * 2;
+  constexpr int WROW = WK == WK_MXFP4 ? KC / 2 : (WK == WK_FP8 ? KC : KC * 2);
   constexpr int LDS_BYTES = 2 * (BM * (KC * 2 + 16) + BN * (WROW + 16));
   GemmParams q = p;
   q.grid_n = (int)cdiv(p.N, BN);
@@ -560,6 +586,17 @@ template <int WK>
 int32_t launch_wk(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st) {
   //                      FM  WM WN MFW NFW KS
   if constexpr (WK == WK_MXFP4) {
+    switch (block_m) {
+      case 16:
+        return launch_cfg<WK, 16, 1, 4, 1, 2, 2>(p, grid_m, swiglu, st);
+      case 32:
+        return launch_cfg<WK, 16, 1, 4, 2, 2, 2>(p, grid_m, swiglu, st);
+      case 64:
+        return launch_cfg<WK, 32, 2, 2, 1, 4, 1>(p, grid_m, swiglu, st);
+      case 128:
+        return launch_cfg<WK, 32, 2, 2, 2, 4, 1>(p, grid_m, swiglu, st);
+    }
+  } else if constexpr (WK == WK_FP8) {
     switch (block_m) {
       case 16:
         return launch_cfg<WK, 16, 1, 4, 1, 2, 2>(p, grid_m, swiglu, st);
@@ -595,17 +632,20 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->M < 0 || d->N < 0 || d->K < 0) return fail(TK_ERR_INVALID, "tk_moe_gemm: negative size");
   if (d->M == 0 || d->N == 0 || d->grid_m == 0) return TK_OK;
   if (!d->x || !d->w || !d->y) return fail(TK_ERR_INVALID, "tk_moe_gemm: null operand");
-  if (d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16 (dtype %d)", d->x_dtype);
+  if (d->x_dtype != TK_BF16 && d->x_dtype != TK_E4M3) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16 or e4m3 (dtype %d)", d->x_dtype);
+  if ((d->x_dtype == TK_E4M3) != (d->w_dtype == TK_E4M3)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: e4m3 activations go with e4m3 weights (x dtype %d, w dtype %d)", d->x_dtype, d->w_dtype);
   if (d->y_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16 (dtype %d)", d->y_dtype);
   if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
   if (d->activation != TK_ACT_NONE && d->activation != TK_ACT_SWIGLU) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad activation %d", d->activation);
   if (d->activation == TK_ACT_SWIGLU && d->N % 2) return fail(TK_ERR_INVALID, "tk_moe_gemm: swiglu needs an even N");
-  if (d->K % 8) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: K must be a multiple of 8 (got %d)", d->K);
-  if (d->x_stride_m % 8 || (reinterpret_cast<uintptr_t>(d->x) & 15)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activation rows must be 16-byte aligned");
+  const int xe = d->x_dtype == TK_E4M3 ? 16 : 8;  // elements per 16 bytes
+  if (d->K % xe) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: K must be a multiple of %d (got %d)", xe, d->K);
+  if (d->x_stride_m % xe || (reinterpret_cast<uintptr_t>(d->x) & 15)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activation rows must be 16-byte aligned");
   if (d->slice_sizes && (!d->slice_offs || !d->block_offs || !d->block_schedule)) return fail(TK_ERR_INVALID, "tk_moe_gemm: incomplete ragged metadata");
   if (d->n_slices >= 65536) return fail(TK_ERR_INVALID, "tk_moe_gemm: at most 65535 slices");
   GemmParams p;
-  p.x = static_cast<const uint16_t*>(d->x);
+  p.x = static_cast<const uint8_t*>(d->x);
+  p.x_is_fp8 = d->x_dtype == TK_E4M3;
   p.x_stride_m = d->x_stride_m;
   p.x_row_scale = d->x_row_scale;
   p.w = static_cast<const uint8_t*>(d->w);
@@ -658,5 +698,12 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     p.w_stride_n = d->w_stride_n * 2;
     return launch_wk<WK_BF16>(p, d->block_m, d->grid_m, swiglu, st);
   }
-  return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weight dtype %d not supported with bf16 activations", d->w_dtype);
+  if (d->w_dtype == TK_E4M3) {
+    if (d->w_mx_scale) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: MX scales with e4m3 weights");
+    if (d->w_stride_n % 16 || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w) & 15)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weight columns must be 16-byte aligned");
+    p.w_stride_e = d->w_stride_e;
+    p.w_stride_n = d->w_stride_n;
+    return launch_wk<WK_FP8>(p, d->block_m, d->grid_m, swiglu, st);
+  }
+  return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weight dtype %d is not supported", d->w_dtype);
 }
