@@ -187,7 +187,7 @@ typedef struct tk_gemm_desc {
   const void* x;
   int32_t x_dtype; /* TK_BF16, or TK_E4M3 with x_row_scale */
   int64_t x_stride_m;
-  const float* x_row_scale; /* fp32 per ROW OF x (indexed after the gather), or NULL */
+  const float* x_row_scale; /* fp32 per row of x, read at the source row src(r), or NULL */
   /* weights: [E, K, N]; e2m1 is packed two per byte along K and the strides count bytes */
   const void* w;
   int32_t w_dtype; /* TK_BF16, TK_E2M1 (needs w_mx_scale), TK_E4M3 */

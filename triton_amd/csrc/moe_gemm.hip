@@ -4,8 +4,8 @@
 //   Y[dst(r), :] = act( (X[src(r), :] @ W[e(r)]) * sx[src(r)] * sw[e(r), :] + bias[e(r), :] ) * gamma[r]
 //
 // Mapping onto CDNA4:
-//   * one workgroup (WM x WN wave64s) computes BM = WM*MFW*16 rows of ONE expert by BN = WN*NFW*16
-//     output columns; the K loop runs in stages of KC = 128*KS;
+//   * one workgroup (WM x WN wave64s) computes BM = WM*MFW*FM rows of ONE expert by BN = WN*NFW*FM
+//     output columns (FM = 16 or 32, the MFMA fragment edge); the K loop runs in stages of KC = 128*KS;
 //   * the MFMA is issued "transposed": the A operand is a 16(n) x 32(k) fragment of W^T and the B
 //     operand a 32(k) x 16(m) fragment of X^T, so a lane's 4 accumulator registers are 4 CONSECUTIVE
 //     output columns of one row (swiglu's (gate, linear) column pairs are lane-local) and both

@@ -2,13 +2,14 @@
 (mirrors the user interface of `triton_kernels/matmul_details/opt_flags.py:20-38,482-603`).
 
 The HIP GEMM is compiled for a fixed set of tile shapes, selected by `block_m` (rows of one expert per
-workgroup):
+workgroup) and the weight format:
 
-    block_m  block_n  block_k  waves   use
-      16       128      256      4     decode: a few rows per expert, weights streamed once
-      32       128      256      4
-      64       256      128      4
-     128       256      128      4     prefill: ~128 rows per expert
+    block_m   mxfp4 / fp8 weights        bf16 weights           use
+              block_n  block_k  waves    block_n  block_k
+      16        128      256      4        128      128         decode: a few rows per expert
+      32        128      256      4        128      128
+      64        256      128      4        128      128
+     128        256      128      4        128      128         prefill: ~128 rows per expert
 
 so only `block_m` can be forced; `block_n`, `block_k` and `num_warps` constraints must match the table.
 `split_k > 1` and `is_persistent=True` cannot be honoured and raise `InapplicableConstraint`, which is
@@ -20,12 +21,21 @@ from contextlib import contextmanager
 from contextvars import ContextVar
 from dataclasses import dataclass
 
-TILE_TABLE = {
+TILE_TABLE = {  # narrow (4-bit / 8-bit) weights
     16: dict(block_n=128, block_k=256, num_warps=4),
     32: dict(block_n=128, block_k=256, num_warps=4),
     64: dict(block_n=256, block_k=128, num_warps=4),
     128: dict(block_n=256, block_k=128, num_warps=4),
 }
+TILE_TABLE_16BIT = {bm: dict(block_n=128, block_k=128, num_warps=4) for bm in TILE_TABLE}
+
+
+def tile_for(block_m: int, rhs_dtype=None) -> dict:
+    """The compiled tile for `block_m` and a weight dtype (torch dtype, package dtype or None = narrow)."""
+    bits = getattr(rhs_dtype, "bitwidth", None)
+    if bits is None:
+        bits = getattr(rhs_dtype, "itemsize", 1) * 8
+    return (TILE_TABLE_16BIT if bits >= 16 else TILE_TABLE)[block_m]
 
 
 @dataclass
@@ -159,7 +169,7 @@ def make_opt_flags(out_dtype, lhs_dtype, rhs_dtype, precision_config, batch_size
     block_m = constraints.get("block_m") or default_block_m(m, ragged_metadata)
     if block_m not in TILE_TABLE:
         raise InapplicableConstraint(f"block_m={block_m} is not one of {sorted(TILE_TABLE)}")
-    tile = TILE_TABLE[block_m]
+    tile = tile_for(block_m, rhs_dtype)
     for key in ("block_n", "block_k", "num_warps"):
         want = constraints.get(key)
         if want is not None and want != tile[key]:
