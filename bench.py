@@ -132,31 +132,64 @@ def cpu_baseline(seed=2):
                 f"{dt:.1f} s wall")
 
 
+def capture(fn):
+    """Captures `fn()` (which returns a tensor) in a HIP graph after a warm-up on a side stream; returns
+    (graph, output tensor that every replay overwrites)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn()
+    return graph, out
+
+
 def bench_decode(device, steps, warmup):
-    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched."""
+    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched.  The whole
+    layer (router, two GEMMs, combine: 6 launches) is replayed from a HIP graph, as a serving loop would; three
+    weight copies are rotated so no step finds its weights in the last-level cache.  Every replay's output is
+    checked against the eager result before timing."""
     E, k, d, f2 = 128, 4, 2880, 5760
     copies = make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)
     per_expert = d * f2 // 2 + d * f2 // 32 + (f2 // 2) * d // 2 + (f2 // 2) * d // 32
     res = {}
     g = torch.Generator().manual_seed(3)
     ebias = torch.randn((E, ), generator=g) * 1.5
-    layer = MoeLayer(copies[0], k)
+    layers = [MoeLayer(w, k) for w in copies]
     for T in (1, 4, 16, 64):
         x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
         logits = (torch.randn((T, E), generator=g) + ebias).to(device)
-        _, rdata = layer(x, logits)
-        active = int((rdata.expt_hist > 0).sum())
+        eager = [layer(x, logits) for layer in layers]
+        active = int((eager[0][1].expt_hist > 0).sum())
         it = [0]
 
-        def step():
-            layer.set_weights(copies[it[0] % len(copies)])  # rotate weight copies: no reuse from the last-level cache
+        def step_eager():
+            layers[it[0] % len(layers)](x, logits)
             it[0] += 1
-            layer(x, logits)
 
-        ms = time_steps(step, steps, warmup)
+        ms_eager = time_steps(step_eager, steps, warmup)
+        graphs = [capture(lambda layer=layer: layer(x, logits)[0]) for layer in layers]
+        for rep in range(2):  # replays with eager work in between, each compared with the eager output
+            for (gr, out), (ref, _) in zip(graphs, eager):
+                gr.replay()
+                torch.cuda.synchronize()
+                if not torch.equal(out, ref):
+                    raise RuntimeError(f"decode T={T}: graph replay {rep} differs from the eager result")
+            step_eager()
+
+        def step_graph():
+            graphs[it[0] % len(graphs)][0].replay()
+            it[0] += 1
+
+        ms = time_steps(step_graph, steps, warmup)
         gbytes = active * per_expert / 1e9
-        res[f"T{T}"] = dict(ms=round(ms, 4), active_experts=active, weight_GB=round(gbytes, 4),
+        res[f"T{T}"] = dict(ms=round(ms, 4), ms_eager=round(ms_eager, 4), active_experts=active, weight_GB=round(gbytes, 4),
                             GBps=round(gbytes / (ms * 1e-3), 1), frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
+        del graphs
     return res
 
 

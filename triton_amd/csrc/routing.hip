@@ -113,6 +113,15 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
       if (p.fill_c) p.fill_c[f] = -1;
     }
   }
+  // the next row's logits are fetched while the current row is being selected
+  float next_v[EPL];
+  if (!p.use_provided_indx && row_begin < row_end && row_begin < n_rows) {
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      next_v[i] = e < E ? load_logit<DT>(p.logits, (int64_t)row_begin * p.stride_m + e) : 0.f;
+    }
+  }
   for (int row = row_begin; row < row_end; ++row) {
     if (row >= n_rows) break;
     float myval = 0.f;
@@ -127,11 +136,13 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
 #pragma unroll
       for (int i = 0; i < EPL; ++i) {
         const int e = lane + 64 * i;
-        if (e < E) {
-          const float v = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e);
-          key[i] = ((unsigned long long)ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e);
-        } else {
-          key[i] = 0ull;
+        key[i] = e < E ? (((unsigned long long)ordered_key(next_v[i]) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
+      }
+      if (row + 1 < row_end && row + 1 < n_rows) {
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const int e = lane + 64 * i;
+          next_v[i] = e < E ? load_logit<DT>(p.logits, (int64_t)(row + 1) * p.stride_m + e) : 0.f;
         }
       }
       for (int j = 0; j < k; ++j) {
@@ -188,101 +199,171 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
 // ---- block-wide exclusive scan (1024 threads) ---------------------------------------------------
 constexpr int kScanThreads = 1024;
 
-__device__ __forceinline__ int block_exclusive_scan(int v, int* total) {
-  __shared__ int wave_sums[kScanThreads / 64 + 1];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int inc = v;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int o = __shfl_up(inc, off);
-    if (lane >= off) inc += o;
-  }
-  __syncthreads();  // protects wave_sums against the previous call's readers
-  if (lane == 63) wave_sums[wave] = inc;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int w = 0; w < kScanThreads / 64; ++w) {
-      const int t = wave_sums[w];
-      wave_sums[w] = run;
-      run += t;
-    }
-    wave_sums[kScanThreads / 64] = run;
-  }
-  __syncthreads();
-  *total = wave_sums[kScanThreads / 64];
-  return inc - v + wave_sums[wave];
-}
-
-// out[i] = sum_{j<i} f(in[j]) for i in [0, n], f(x) = ceil(x / 2^shift)
-__device__ __forceinline__ void scan_to(const int32_t* in, int n, int shift, int32_t* out) {
-  int carry = 0;
-  for (int base = 0; base < n; base += kScanThreads) {
-    const int i = base + threadIdx.x;
-    int v = 0;
-    if (i < n) v = (in[i] + ((1 << shift) - 1)) >> shift;
-    int total;
-    const int ex = block_exclusive_scan(v, &total);
-    if (i < n) out[i] = carry + ex;
-    carry += total;
-  }
-  if (threadIdx.x == 0) out[n] = carry;
-}
-
 struct RaggedOut {
-  int32_t* slice_offs;    // [E+1]
-  int32_t* block_offs;    // [kNumBlockSizes][stride]
+  int32_t* slice_offs;    // [E+1] or null
+  int32_t* block_offs;    // [kNumBlockSizes][stride] or null
   int64_t block_offs_stride;
   int32_t* block_sched;   // [kNumBlockSizes][stride]
   int64_t block_sched_stride;
   int32_t max_n_blocks;
 };
 
-__device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int E, const RaggedOut r) {
-  scan_to(slice_sizes, E, 0, r.slice_offs);
-  for (int b = 0; b < kNumBlockSizes; ++b)
-    scan_to(slice_sizes, E, kFirstBlockLog2 + b, r.block_offs + b * r.block_offs_stride);
-  for (int b = 0; b < kNumBlockSizes; ++b)
-    for (int i = threadIdx.x; i < r.max_n_blocks; i += kScanThreads) r.block_sched[b * r.block_sched_stride + i] = -1;
+constexpr int kScanWaves = kScanThreads / 64;
+constexpr int kQuantities = 1 + kNumBlockSizes;  // rows, then row blocks of 16, 32, 64, 128, 256
+
+// Exclusive scans of the slice sizes and of their block counts for all block sizes in ONE pass over the
+// slices: each thread carries the six quantities of its slice through a wave scan, the wave totals are
+// exchanged once through LDS.  offs0 (optional) and r.slice_offs (optional) receive the row offsets,
+// r.block_offs the block offsets.  Then every schedule slot finds its slice by binary search in the
+// block offsets, so a slice with thousands of blocks costs no more than an empty one.
+__device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int E, int32_t* offs0, const RaggedOut r, bool want_ragged) {
+  __shared__ int wave_tot[kQuantities][kScanWaves + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nq = want_ragged ? kQuantities : 1;
+  int carry[kQuantities];
+#pragma unroll
+  for (int q = 0; q < kQuantities; ++q) carry[q] = 0;
+  for (int base = 0; base < E; base += kScanThreads) {
+    const int i = base + threadIdx.x;
+    const int sz = i < E ? slice_sizes[i] : 0;
+    int v[kQuantities], inc[kQuantities];
+    v[0] = sz;
+#pragma unroll
+    for (int b = 0; b < kNumBlockSizes; ++b) v[1 + b] = (sz + ((1 << (kFirstBlockLog2 + b)) - 1)) >> (kFirstBlockLog2 + b);
+#pragma unroll
+    for (int q = 0; q < kQuantities; ++q) {
+      inc[q] = v[q];
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int o = __shfl_up(inc[q], off);
+        if (lane >= off) inc[q] += o;
+      }
+    }
+    __syncthreads();  // wave_tot may still be read by the previous trip
+    if (lane == 63) {
+#pragma unroll
+      for (int q = 0; q < kQuantities; ++q) wave_tot[q][wave] = inc[q];
+    }
+    __syncthreads();
+    if (threadIdx.x < kQuantities) {
+      int run = 0;
+      for (int w = 0; w < kScanWaves; ++w) {
+        const int t = wave_tot[threadIdx.x][w];
+        wave_tot[threadIdx.x][w] = run;
+        run += t;
+      }
+      wave_tot[threadIdx.x][kScanWaves] = run;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kQuantities; ++q) {
+      if (q < nq && i < E) {
+        const int ex = carry[q] + wave_tot[q][wave] + inc[q] - v[q];
+        if (q == 0) {
+          if (offs0) offs0[i] = ex;
+          if (want_ragged) r.slice_offs[i] = ex;
+        } else {
+          r.block_offs[(q - 1) * r.block_offs_stride + i] = ex;
+        }
+      }
+      carry[q] += wave_tot[q][kScanWaves];
+    }
+  }
+  if (threadIdx.x == 0) {
+    if (offs0) offs0[E] = carry[0];
+    if (want_ragged) {
+      r.slice_offs[E] = carry[0];
+#pragma unroll
+      for (int b = 0; b < kNumBlockSizes; ++b) r.block_offs[b * r.block_offs_stride + E] = carry[1 + b];
+    }
+  }
+  if (!want_ragged) return;
   __threadfence_block();
   __syncthreads();
+#pragma unroll
   for (int b = 0; b < kNumBlockSizes; ++b) {
-    const int shift = kFirstBlockLog2 + b;
     const int32_t* offs = r.block_offs + b * r.block_offs_stride;
     int32_t* sched = r.block_sched + b * r.block_sched_stride;
-    for (int e = threadIdx.x; e < E; e += kScanThreads) {
-      const int nb = (slice_sizes[e] + ((1 << shift) - 1)) >> shift;
-      const int o = offs[e];
-      for (int j = 0; j < nb; ++j)
-        if (o + j < r.max_n_blocks) sched[o + j] = (j << 16) | e;
+    const int total = carry[1 + b];
+    for (int i = threadIdx.x; i < r.max_n_blocks; i += kScanThreads) {
+      int val = -1;
+      if (i < total) {
+        int lo = 0, hi = E;  // largest e with offs[e] <= i; empty slices share an offset, the last one wins
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (offs[mid] <= i) lo = mid; else hi = mid;
+        }
+        val = ((i - offs[lo]) << 16) | lo;
+      }
+      sched[i] = val;
     }
   }
 }
 
+// Exclusive prefix over the waves' histograms, per expert.  Threads are laid out [group][expert] so that a
+// wave reads consecutive experts of one unit (coalesced); the units are split into `groups` contiguous
+// runs that are summed in parallel (pass 1), offset by an LDS exchange of the run totals, and rewritten
+// as exclusive prefixes (pass 2) with the loads of a chunk issued before its dependent stores.
 __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* partials, int units, int E, int32_t* col_sum,
                                                                   int32_t* col_offs, int want_ragged, const RaggedOut r) {
-  for (int e = threadIdx.x; e < E; e += kScanThreads) {
-    int run = 0;
-    for (int u = 0; u < units; ++u) {
-      const int64_t i = (int64_t)u * E + e;
-      const int t = partials[i];
-      partials[i] = run;
-      run += t;
+  __shared__ int32_t run_total[kScanThreads];
+  int groups = kScanThreads / E;
+  groups = groups < 1 ? 1 : (groups > 32 ? 32 : groups);
+  groups = groups > units ? units : groups;
+  const int per_group = (units + groups - 1) / groups;
+  constexpr int kChunk = 8;
+  for (int e0 = 0; e0 < E; e0 += kScanThreads) {  // more than one trip only when E > 1024 (then groups == 1)
+    const int e = e0 + (int)(threadIdx.x % (unsigned)(E < kScanThreads ? E : kScanThreads));
+    const int g = (int)(threadIdx.x / (unsigned)(E < kScanThreads ? E : kScanThreads));
+    const bool active = e < E && g < groups;
+    const int u_begin = g * per_group;
+    int u_end = u_begin + per_group;
+    u_end = u_end < units ? u_end : units;
+    int sum = 0;
+    if (active) {
+      int u = u_begin;
+      for (; u + kChunk <= u_end; u += kChunk) {
+        int v[kChunk];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) v[i] = partials[(int64_t)(u + i) * E + e];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) sum += v[i];
+      }
+      for (; u < u_end; ++u) sum += partials[(int64_t)u * E + e];
     }
-    col_sum[e] = run;
+    __syncthreads();  // run_total may still be read by the previous trip
+    if (active) run_total[threadIdx.x] = sum;
+    __syncthreads();
+    if (active) {
+      const int width = E < kScanThreads ? E : kScanThreads;
+      int run = 0;
+      for (int gg = 0; gg < g; ++gg) run += run_total[gg * width + (e - e0)];
+      int u = u_begin;
+      for (; u + kChunk <= u_end; u += kChunk) {
+        int v[kChunk];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) v[i] = partials[(int64_t)(u + i) * E + e];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) {
+          partials[(int64_t)(u + i) * E + e] = run;
+          run += v[i];
+        }
+      }
+      for (; u < u_end; ++u) {
+        const int t = partials[(int64_t)u * E + e];
+        partials[(int64_t)u * E + e] = run;
+        run += t;
+      }
+      if (g == groups - 1) col_sum[e] = run;
+    }
   }
   __threadfence_block();
   __syncthreads();
-  scan_to(col_sum, E, 0, col_offs);
-  if (want_ragged) {
-    __threadfence_block();
-    __syncthreads();
-    ragged_metadata(col_sum, E, r);
-  }
+  ragged_metadata(col_sum, E, col_offs, r, want_ragged != 0);
 }
 
 __global__ __launch_bounds__(kScanThreads) void ragged_metadata_kernel(const int32_t* slice_sizes, int E, const RaggedOut r) {
-  ragged_metadata(slice_sizes, E, r);
+  ragged_metadata(slice_sizes, E, nullptr, r, true);
 }
 
 struct ScatterParams {
@@ -349,8 +430,11 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
   }
 }
 
+// Rows one wave routes: one for small batches (latency), more as T grows so that the per-wave
+// histograms the scan has to walk stay at <= 256 rows of the workspace up to T = 4096 (<= 1024 beyond).
 int rows_per_wave_for(int T) {
-  int rpw = 16;
+  int rpw = 1;
+  while ((int64_t)rpw * 256 < T && rpw < 16) rpw *= 2;
   while ((int64_t)rpw * 1024 < T) rpw *= 2;
   return rpw;
 }
