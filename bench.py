@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+# HBM bytes one launch of the first expert GEMM moves at this workload, from two counter runs over this script
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from the 1 GiB copy of --calibrate-copy): 1819.1 MB read
+# + 103.1 MB written, against 1318.3 MB of algorithmic bytes.
+GEMM1_TRAFFIC_BYTES = 1.922e9
 
 
 def make_moe_weights(E, d_model, d_ff2, seed, device, n_copies=1):
@@ -106,12 +110,12 @@ def time_steps(fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def cpu_baseline(seed=2):
-    """CPU oracle on a bounded sample of config 3: 16 of the 128 experts and 512 tokens (top-4), which
-    keeps the ~128 routed rows per expert of the full workload."""
+def cpu_baseline(seed=2, min_seconds=10.0):
+    """CPU oracle on a bounded sample of config 3: 32 of the 128 experts and 1024 tokens (top-4), which keeps
+    the ~128 routed rows per expert of the full workload; passes are repeated until `min_seconds` of CPU work."""
     from oracle import moe as omoe
     from oracle import mxfp as omx
-    E, T, k, d, f2 = 16, 512, 4, 2880, 5760
+    E, T, k, d, f2 = 32, 1024, 4, 2880, 5760
     g = torch.Generator().manual_seed(seed)
     x = torch.randn((T, d), generator=g).to(torch.bfloat16)
     logits = torch.randn((T, E), generator=g)
@@ -122,14 +126,28 @@ def cpu_baseline(seed=2):
     w1q, w1s = omx.downcast_to_mxfp(w1, torch.uint8, axis=1)
     w2q, w2s = omx.downcast_to_mxfp(w2, torch.uint8, axis=1)
     del w1, w2
-    torch.set_num_threads(os.cpu_count() or 1)
-    t0 = time.perf_counter()
-    omoe.moe_layer(x, logits, k, w1q, b1, w2q, b2, w1_mx_scale=w1s, w2_mx_scale=w2s)
-    dt = time.perf_counter() - t0
-    flops = 2.0 * T * k * d * (f2 + d)
-    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"CPU oracle (oracle/moe.py) on {E} of 128 experts x {T} tokens, top-{k}, same per-expert shapes; "
-                f"{dt:.1f} s wall")
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        omoe.moe_layer(x, logits, k, w1q, b1, w2q, b2, w1_mx_scale=w1s, w2_mx_scale=w2s)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds or passes >= 20:
+            break
+    flops = 2.0 * T * k * d * (f2 + d) * passes
+    return dict(value=round(flops / dt / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"CPU oracle (oracle/moe.py: dequantise MXFP4, fp32 torch.matmul per expert) on {E} of 128 experts x {T} "
+                f"tokens, top-{k}, same per-expert shapes; {passes} passes in {dt:.1f} s wall")
+
+
+def calibration_copy(device, reps=3):
+    """A copy of known size (1 GiB read + 1 GiB written per launch) so that a counter run over this script
+    holds a kernel whose FETCH_SIZE / WRITE_SIZE readings can be compared with its true bytes."""
+    src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(reps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
 
 
 def capture(fn):
@@ -213,6 +231,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the decode and MX round-trip figures")
+    ap.add_argument("--calibrate-copy", action="store_true", help="also run a 1 GiB device copy (reference kernel for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (expert-parallel sharding is described in DESIGN.md)",
@@ -229,6 +248,8 @@ def main():
     logits = torch.randn((T, E), generator=g).to(device)
     weights = make_moe_weights(E, d, f2, seed=2, device=device)[0]
     layer = MoeLayer(weights, k)
+    if args.calibrate_copy:
+        calibration_copy(device)
 
     for _ in range(args.warmup):
         layer(x, logits)
@@ -262,7 +283,7 @@ def main():
         "config": {"workload": "gpt-oss-120b-shaped MXFP4 MoE FFN prefill (BASELINE config 3)", "tokens": T, "d_model": d,
                    "experts": E, "top_k": k, "w1": [E, d, f2], "w2": [E, f2 // 2, d]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM1_TRAFFIC_BYTES,
                      "kernel": "moe_gemm_kernel (gather-GEMM W1 + bias + swiglu)", "kernel_ms": round(gemm1_ms, 4)},
     }
     # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
