@@ -165,6 +165,21 @@ int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t
  * Ragged expert GEMM
  * ---------------------------------------------------------------------------------------------- */
 
+/*
+ * How `w` / `w_mx_scale` are laid out.  TK_W_STRIDED is the reference's strided form (what
+ * `downcast_to_mxfp(w, uint8, axis=1)` returns, tk/numerics_details/mxfp.py:61-64).  TK_W_TILED is this
+ * library's pre-tiled MXFP4 form, the counterpart of the reference's architecture-specific weight layouts
+ * (tk/tensor_details/layout.py:26-54, built once per model with `convert_layout`): per expert, per fragment
+ * F of 32 output columns (N padded to 32), per K-stage s of 128 (K padded to 128, zero weights):
+ *   values  one 2048-byte block at ((F * S + s) * 2048), S = ceil(K / 128), ordered [q:2][lane:64][16 bytes];
+ *           lane = h*32 + c holds the packed e2m1 bytes (even k in the low nibble) of column F*32 + c for
+ *           k in [s*128 + h*64 + q*32, +32);
+ *   scales  one 128-byte block at ((F * S + s) * 128) ordered [c:32][4]: the four e8m0 bytes of column
+ *           F*32 + c for the stage's four 32-element blocks.
+ * The w_stride_e / ws_stride_e fields give the bytes from one expert to the next; the k / n strides are unused.
+ */
+enum tk_w_layout { TK_W_STRIDED = 0, TK_W_TILED = 1 };
+
 enum tk_activation {
   TK_ACT_NONE = 0,
   TK_ACT_SWIGLU = 1 /* interleaved (gate, linear) columns -> N/2 outputs, tk/swiglu_details/_swiglu.py:55-70 */
@@ -222,6 +237,7 @@ typedef struct tk_gemm_desc {
   int32_t activation; /* enum tk_activation */
   float act_alpha, act_limit;
   int32_t act_has_limit;
+  int32_t w_layout; /* enum tk_w_layout */
 } tk_gemm_desc;
 
 /* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */

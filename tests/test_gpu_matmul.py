@@ -34,9 +34,15 @@ def _slice_sizes(m, n_slices, g):
 
 def _make_w(E, K, N, kind, g, device):
     w = (torch.randn((E, K, N), generator=g) * 0.5 / K**0.5 * 4).to(torch.bfloat16)
-    if kind == "mxfp4":
+    if kind in ("mxfp4", "mxfp4_tiled"):
         q, s = omx.downcast_to_mxfp(w, torch.uint8, axis=1)
-        return dict(w_dev=q.to(device), scale_dev=s.to(device), w_cpu=q, scale_cpu=s)
+        qd, sd = q.to(device), s.to(device)
+        if kind == "mxfp4_tiled":  # the pre-tiled layouts, converted as the reference converts its weight layouts
+            from triton_amd.tensor import FP4, convert_layout, wrap_torch_tensor
+            from triton_amd.tensor_details.layout import make_default_matmul_mxfp4_w_layout, make_default_matmul_mxfp4_w_scale_layout
+            qd = convert_layout(wrap_torch_tensor(qd, dtype=FP4), make_default_matmul_mxfp4_w_layout(mx_axis=1))
+            sd = convert_layout(wrap_torch_tensor(sd), make_default_matmul_mxfp4_w_scale_layout(mx_axis=1))
+        return dict(w_dev=qd, scale_dev=sd, w_cpu=q, scale_cpu=s)
     if kind == "bf16_kmajor":
         wd = w.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)
         return dict(w_dev=wd, scale_dev=None, w_cpu=w, scale_cpu=None)
@@ -54,11 +60,16 @@ CASES = [
     (720, 576, 768, "plain", "mxfp4"),
     (600, 400, 416, "plain", "bf16"),
     (5, 2880, 2880, "ragged", "mxfp4"),
+    (300, 400, 416, "ragged", "mxfp4_tiled"),
+    (720, 576, 768, "ragged", "mxfp4_tiled"),
+    (1500, 512, 1024, "ragged", "mxfp4_tiled"),
+    (720, 576, 768, "plain", "mxfp4_tiled"),
+    (5, 2880, 2880, "ragged", "mxfp4_tiled"),
 ]
 
 
 @pytest.mark.parametrize("m, n, k, mode, wkind", CASES)
-@pytest.mark.parametrize("block_m", [16, 128])
+@pytest.mark.parametrize("block_m", [16, 64, 128])
 @pytest.mark.parametrize("do_gather, do_scatter", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("do_gamma", [False, True])
 def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatter, do_gamma):
@@ -87,11 +98,12 @@ def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatt
         written = torch.zeros(m, dtype=torch.bool)
         written[scatter[scatter >= 0].long()] = True
         got = torch.where(written[:, None], got, torch.zeros_like(got))
-    assert_close(ref, got, maxtol=3e-2 if wkind == "mxfp4" else 2e-2, what="y")
+    assert_close(ref, got, maxtol=3e-2 if wkind.startswith("mxfp4") else 2e-2, what="y")
     assert_allclose_gate(ref, got, what="y")
 
 
-@pytest.mark.parametrize("m, n, k, wkind", [(300, 512, 416, "bf16_kmajor"), (720, 576, 768, "mxfp4"), (40, 5760, 2880, "mxfp4")])
+@pytest.mark.parametrize("m, n, k, wkind", [(300, 512, 416, "bf16_kmajor"), (720, 576, 768, "mxfp4"), (40, 5760, 2880, "mxfp4"),
+                                            (720, 576, 768, "mxfp4_tiled"), (900, 5760, 2880, "mxfp4_tiled")])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])
 @pytest.mark.parametrize("opts", [(1.1, 1.4), (1.702, 7.0), (0.5, None)])
 def test_fused_swiglu(mods, device, m, n, k, wkind, block_m, opts):

@@ -34,6 +34,7 @@ _c = ctypes
 _i32, _i64, _ptr, _f32 = _c.c_int32, _c.c_int64, _c.c_void_p, _c.c_float
 
 TK_ACT_NONE, TK_ACT_SWIGLU = 0, 1
+TK_W_STRIDED, TK_W_TILED = 0, 1
 
 
 class RouteDesc(_c.Structure):
@@ -62,6 +63,7 @@ class GemmDesc(_c.Structure):
         ("n_slices", _i32), ("block_m", _i32), ("grid_m", _i32), ("M", _i32), ("N", _i32), ("K", _i32),
         ("y", _ptr), ("y_dtype", _i32), ("y_stride_m", _i64),
         ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
+        ("w_layout", _i32),
     ]
 
 

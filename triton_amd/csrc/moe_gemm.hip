@@ -26,6 +26,17 @@
 namespace tk {
 namespace {
 
+// f(integral_constant<int, I>) for I in [B, E), fully expanded at compile time
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3
 
 struct GemmParams {
@@ -62,6 +73,7 @@ struct GemmParams {
   int32_t has_limit;
   int32_t y_vec;     // output rows allow 16-byte vector stores
   int32_t bias_vec;  // bias rows allow 16-byte vector loads
+  int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
 };
 
 __device__ inline int xcd_remap(int pid, int total) {
@@ -125,6 +137,161 @@ struct Frag<32> {
   }
   static __device__ __forceinline__ int n_of(int i, int h) { return (i >> 2) * 8 + h * 4 + (i & 3); }
 };
+
+// Epilogue shared by the GEMM kernels.  acc[f][j] is the FM x FM fragment of column fragment f (first column
+// ncol0 + f*FM) and row fragment j (tile rows (j*WM + mw)*FM ..); register i of a lane in lane group h holds
+// output column Frag::n_of(i, h) of row lr.  Order: row/column scales, bias, activation, gate weight,
+// (scattered) store.  Everything the rows and columns need from memory is fetched before the first store.
+template <int FM, int WM, int MFW, int NFW, bool SWIGLU>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag<FM>::acc_t (&acc)[NFW][MFW], int expert,
+                                              int off_m, int start_m, int eM, int ncol0, bool full_n, int mw, int lr, int h) {
+  typedef Frag<FM> FR;
+  const int N = p.N;
+  const int NOUT = SWIGLU ? N / 2 : N;
+  // per-row items; rows past the slice read the slice's last row (no divergent branches around the loads)
+  float gam[MFW], rsc[MFW];
+  int64_t dst[MFW];
+  bool ok[MFW];
+  int srow[MFW];
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const int row = off_m + (j * WM + mw) * FM + lr;  // row inside the slice
+    ok[j] = row < eM;
+    srow[j] = start_m + (ok[j] ? row : eM - 1);       // row in expert-sorted order
+    gam[j] = 1.0f;
+    rsc[j] = 1.0f;
+    dst[j] = srow[j];
+  }
+  if (p.gammas) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) gam[j] = load_scalar(p.gammas, srow[j], p.gammas_is_f32);
+  }
+  if (p.scatter) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) {
+      const int sr = srow[j] < p.scatter_len ? srow[j] : p.scatter_len - 1;
+      const int v = p.scatter[sr];
+      dst[j] = srow[j] < p.scatter_len ? v : -1;
+    }
+  }
+  if (p.x_row_scale) {
+    int src[MFW];
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) src[j] = p.gather ? p.gather[srow[j]] : srow[j];
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) rsc[j] = p.x_row_scale[src[j]];
+  }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) ok[j] = ok[j] && dst[j] >= 0;
+  if (p.x_row_scale || p.w_col_scale) {  // fp8-style per-row x per-column scales
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int i = 0; i < FR::NACC; ++i) {
+        const int n = ncol0 + f * FM + FR::n_of(i, h);
+        float cs = 1.0f;
+        if (p.w_col_scale && n < N) cs = p.w_col_scale[expert * p.wcs_stride_e + n];
+#pragma unroll
+        for (int j = 0; j < MFW; ++j) acc[f][j][i] *= rsc[j] * cs;
+      }
+  }
+  if (p.bias) {
+    float b4[NFW][FR::NACC / 4][4];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int q = 0; q < FR::NACC / 4; ++q) {
+        const int n0 = ncol0 + f * FM + FR::n_of(4 * q, h);  // 4 consecutive columns
+        const int64_t bo = expert * p.bias_stride_e + n0;
+        if (full_n && p.bias_vec) {
+          if (p.bias_is_f32) {
+            const float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(p.bias) + bo);
+            b4[f][q][0] = t.x, b4[f][q][1] = t.y, b4[f][q][2] = t.z, b4[f][q][3] = t.w;
+          } else {
+            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p.bias) + bo);
+            b4[f][q][0] = bits_f32(t.x << 16), b4[f][q][1] = bits_f32(t.x & 0xFFFF0000u);
+            b4[f][q][2] = bits_f32(t.y << 16), b4[f][q][3] = bits_f32(t.y & 0xFFFF0000u);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) b4[f][q][i] = n0 + i < N ? load_scalar(p.bias, bo + i, p.bias_is_f32) : 0.f;
+        }
+      }
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int q = 0; q < FR::NACC / 4; ++q)
+#pragma unroll
+        for (int j = 0; j < MFW; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] += b4[f][q][i];
+  }
+  // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
+  // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
+  constexpr int VW = FM == 32 ? 8 : 4;
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    uint16_t* yrow = p.y + (ok[j] ? dst[j] : 0) * p.y_stride_m;
+    const float g = gam[j];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) {
+#pragma unroll
+      for (int u = 0; u < FR::NACC / VW; ++u) {
+        float v[VW];
+        int n0;
+        if constexpr (FM == 32) {
+          // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint32_t lo = f32_bits(acc[f][j][8 * u + i]), hi = f32_bits(acc[f][j][8 * u + 4 + i]);
+            auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo's upper half <-> hi's lower half
+            v[i] = bits_f32(r[0]);
+            v[4 + i] = bits_f32(r[1]);
+          }
+          n0 = ncol0 + f * FM + 16 * u + 8 * h;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = acc[f][j][4 * u + i];
+          n0 = ncol0 + f * FM + FR::n_of(4 * u, h);
+        }
+        if (!ok[j]) continue;
+        if (SWIGLU) {
+          float r[VW / 2];
+#pragma unroll
+          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[2 * i], v[2 * i + 1], p.alpha, p.limit, p.has_limit) * g;
+          const int o0 = n0 / 2;
+          if (o0 + VW / 2 <= NOUT && p.y_vec) {
+            uint32_t w[VW / 4];
+#pragma unroll
+            for (int i = 0; i < VW / 4; ++i) w[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint2*>(yrow + o0) = make_uint2(w[0], w[VW / 4 - 1]);
+            else
+              *reinterpret_cast<uint32_t*>(yrow + o0) = w[0];
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i)
+              if (o0 + i < NOUT) yrow[o0 + i] = f32_to_bf16_bits(r[i]);
+          }
+        } else {
+          if (n0 + VW <= N && p.y_vec) {
+            uint32_t w[VW / 2];
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[2 * i] * g, v[2 * i + 1] * g);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint4*>(yrow + n0) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
+            else
+              *reinterpret_cast<uint2*>(yrow + n0) = make_uint2(w[0], w[1]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW; ++i)
+              if (n0 + i < N) yrow[n0 + i] = f32_to_bf16_bits(v[i] * g);
+          }
+        }
+      }
+    }
+  }
+}
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS, bool SWIGLU>
 __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams p) {
@@ -430,130 +597,256 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
     __syncthreads();
   }
 
-  // ---- epilogue ------------------------------------------------------------------------------
-  // order: row/column scales, bias, activation, gate weight, (scattered) store
-  const int NOUT = SWIGLU ? N / 2 : N;
-  const bool full_n = n_tile + BN <= N;
-  if (p.x_row_scale || p.w_col_scale) {  // fp8-style per-row x per-column scales (rare path)
-#pragma unroll
-    for (int j = 0; j < MFW; ++j) {
-      const int row = off_m + (j * WM + mw) * FM + lr;
-      float rs = 1.0f;
-      if (p.x_row_scale && row < eM) rs = p.x_row_scale[p.gather ? p.gather[start_m + row] : start_m + row];
-#pragma unroll
-      for (int f = 0; f < NFW; ++f)
-#pragma unroll
-        for (int i = 0; i < FR::NACC; ++i) {
-          const int n = n_tile + (nw * NFW + f) * FM + FR::n_of(i, h);
-          float cs = 1.0f;
-          if (p.w_col_scale && n < N) cs = p.w_col_scale[expert * p.wcs_stride_e + n];
-          acc[f][j][i] *= rs * cs;
-        }
-    }
+  gemm_epilogue<FM, WM, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, n_tile + nw * NFW * FM, n_tile + BN <= N, mw, lr, h);
+}
+
+// ------------------------------------------------------------------------------------------------
+// MXFP4 weights in the tile-native layout (prefill: block_m 64 / 128)
+// ------------------------------------------------------------------------------------------------
+// Weight layout (built once per model by the host from the K-contiguous form): per expert, per fragment F of
+// 32 output columns, per K-stage s of 128: one 2 KiB block [q:2][lane:64][16 B]; lane = h*32 + lr holds the
+// packed e2m1 bytes of column F*32 + lr for k in [s*128 + h*64 + q*32, +32).  Scales: one 128 B block
+// [lr:32][4] per (F, s) with the four e8m0 bytes of column lr's stage.  N is padded to 32 and K to 128 with
+// zero weights.  A wave owns two column fragments and reads its weights straight from global memory into
+// registers (every load instruction fetches 1 KiB contiguous, nothing is shared between waves, so they
+// bypass LDS); only the gathered activation rows, which all four waves need, are staged through LDS.
+//
+// Pipeline per K-stage (8 MFMA steps of k = 16): the MFMAs of step t are interleaved, in program order pinned
+// by scheduling barriers, with the LDS reads and e2m1 -> bf16 conversions of step t+1, with the LDS writes of
+// the next stage's activations and the global loads of the stage after it.  One workgroup barrier per stage
+// sits in step 7, after every wave has fetched its last operands of the current LDS buffer.
+template <int MFW, bool SWIGLU>
+__global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
+  typedef Frag<32> FR;
+  constexpr int FM = 32, NFW = 2, NT = 256, BM = MFW * 32, BN = 256, KC = 128;
+  constexpr int XPITCH = KC * 2 + 16;
+  constexpr int XBYTES = BM * XPITCH;
+  constexpr int XCH = BM * 16 / NT;  // 16-byte activation pieces per thread per stage (4 or 8)
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  int expert, off_m, start_m, eM, pid_n;
+  if (p.slice_sizes) {
+    const int live = p.block_offs[p.n_slices] * p.grid_n;
+    if ((int)blockIdx.x >= live) return;
+    const int pid = xcd_remap(blockIdx.x, live);
+    pid_n = pid % p.grid_n;
+    const int sched = p.block_sched[pid / p.grid_n];
+    expert = sched & 0xFFFF;
+    off_m = (sched >> 16) * BM;
+    start_m = p.slice_offs[expert];
+    eM = p.slice_sizes[expert];
+  } else {
+    const int pid = xcd_remap(blockIdx.x, gridDim.x);
+    pid_n = pid % p.grid_n;
+    expert = 0;
+    off_m = (pid / p.grid_n) * BM;
+    start_m = 0;
+    eM = p.M;
   }
-  if (p.bias) {
+  const int rows = (eM - off_m) < BM ? (eM - off_m) : BM;
+  const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW)
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int nw = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 31, h = lane >> 5;
+  const int K = p.K, N = p.N;
+  const int nst = p.w_nst;
+
+  // ---- activation staging: this thread's 16-byte pieces (row r_j = tid/16 + 16 j, k-chunk c = tid%16) ----
+  const int xc = tid & 15;
+  const uint8_t* xptr[XCH];
 #pragma unroll
-    for (int f = 0; f < NFW; ++f)
-#pragma unroll
-      for (int q = 0; q < FR::NACC / 4; ++q) {
-        const int n0 = n_tile + (nw * NFW + f) * FM + FR::n_of(4 * q, h);  // 4 consecutive columns
-        float b4[4];
-        const int64_t bo = expert * p.bias_stride_e + n0;
-        if (full_n && p.bias_vec) {
-          if (p.bias_is_f32) {
-            const float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(p.bias) + bo);
-            b4[0] = t.x, b4[1] = t.y, b4[2] = t.z, b4[3] = t.w;
-          } else {
-            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p.bias) + bo);
-            b4[0] = bits_f32(t.x << 16), b4[1] = bits_f32(t.x & 0xFFFF0000u);
-            b4[2] = bits_f32(t.y << 16), b4[3] = bits_f32(t.y & 0xFFFF0000u);
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) b4[i] = n0 + i < N ? load_scalar(p.bias, bo + i, p.bias_is_f32) : 0.f;
-        }
-#pragma unroll
-        for (int j = 0; j < MFW; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] += b4[i];
-      }
+  for (int j = 0; j < XCH; ++j) {
+    const int r = (tid >> 4) + 16 * j;
+    int row = off_m + r;
+    row = row < eM ? row : eM - 1;
+    const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
+    xptr[j] = p.x + src * p.x_stride_m * 2;  // the k offset (incl. this thread's chunk) is added per stage
   }
-  // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
-  // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
-  constexpr int VW = FM == 32 ? 8 : 4;
+  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // piece j at xlds0 + j*16*XPITCH
+
+  // ---- weights: two column fragments of this wave ----
+  const int nfr = (N + 31) >> 5;
+  const uint8_t* wptr[NFW];
+  const uint8_t* sptr[NFW];
 #pragma unroll
-  for (int j = 0; j < MFW; ++j) {
-    const int row = off_m + (j * WM + mw) * FM + lr;  // row inside the slice
-    const int srow = start_m + row;                   // row in expert-sorted order
-    bool ok = row < eM;
-    float gam = 1.0f;
-    int64_t dst = srow;
-    if (ok) {
-      if (p.gammas) gam = load_scalar(p.gammas, srow, p.gammas_is_f32);
-      if (p.scatter) {
-        dst = srow < p.scatter_len ? p.scatter[srow] : -1;
-        ok = dst >= 0;
-      }
-    }
-    uint16_t* yrow = p.y + (ok ? dst : 0) * p.y_stride_m;
+  for (int f = 0; f < NFW; ++f) {
+    int F = pid_n * (BN / 32) + nw * NFW + f;
+    F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
+    wptr[f] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 2048 + lane * 16;
+    sptr[f] = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)F * nst * 128 + lr * 4;
+  }
+
+  typename FR::acc_t acc[NFW][MFW];
+#pragma unroll
+  for (int f = 0; f < NFW; ++f)
+#pragma unroll
+    for (int j = 0; j < MFW; ++j)
+#pragma unroll
+      for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
+
+  u32x4_t xreg[XCH];  // native vectors: arrays of the HIP uint4 struct were left in scratch memory here
+  u32x4_t wraw[2][NFW][2];
+  uint32_t sd[2][NFW];
+  bf16x8_t xf[2][MFW];
+  bf16x8_t wf[2][NFW];
+
+  // Loads are unconditional (no divergent control flow inside the pipeline): rows past the tile's last
+  // valid row re-read that row, k past K re-reads the row's last 8 values (the padded weights there are
+  // zero), stages past the last one re-read the last stage.
+  auto load_x_piece = [&](int j, int s) __attribute__((always_inline)) {
+    int k0 = s * KC + xc * 8;
+    k0 = k0 < K - 8 ? k0 : K - 8;
+    xreg[j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0 * 2);
+  };
+  auto store_x_piece = [&](int j, int buf) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 16 * XPITCH) = xreg[j];
+  };
+  auto load_w = [&](auto par_c, int s) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_c)::value;
+    s = s < nst ? s : nst - 1;
 #pragma unroll
     for (int f = 0; f < NFW; ++f) {
-#pragma unroll
-      for (int u = 0; u < FR::NACC / VW; ++u) {
-        float v[VW];
-        int n0;
-        if constexpr (FM == 32) {
-          // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            uint32_t lo = f32_bits(acc[f][j][8 * u + i]), hi = f32_bits(acc[f][j][8 * u + 4 + i]);
-            auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo's upper half <-> hi's lower half
-            v[i] = bits_f32(r[0]);
-            v[4 + i] = bits_f32(r[1]);
-          }
-          n0 = n_tile + (nw * NFW + f) * FM + 16 * u + 8 * h;
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = acc[f][j][4 * u + i];
-          n0 = n_tile + (nw * NFW + f) * FM + FR::n_of(4 * u, h);
-        }
-        if (!ok) continue;
-        if (SWIGLU) {
-          float r[VW / 2];
-#pragma unroll
-          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[2 * i], v[2 * i + 1], p.alpha, p.limit, p.has_limit) * gam;
-          const int o0 = n0 / 2;
-          if (o0 + VW / 2 <= NOUT && p.y_vec) {
-            uint32_t w[VW / 4];
-#pragma unroll
-            for (int i = 0; i < VW / 4; ++i) w[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
-            if constexpr (VW == 8)
-              *reinterpret_cast<uint2*>(yrow + o0) = make_uint2(w[0], w[VW / 4 - 1]);
-            else
-              *reinterpret_cast<uint32_t*>(yrow + o0) = w[0];
-          } else {
-#pragma unroll
-            for (int i = 0; i < VW / 2; ++i)
-              if (o0 + i < NOUT) yrow[o0 + i] = f32_to_bf16_bits(r[i]);
-          }
-        } else {
-          if (n0 + VW <= N && p.y_vec) {
-            uint32_t w[VW / 2];
-#pragma unroll
-            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[2 * i] * gam, v[2 * i + 1] * gam);
-            if constexpr (VW == 8)
-              *reinterpret_cast<uint4*>(yrow + n0) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
-            else
-              *reinterpret_cast<uint2*>(yrow + n0) = make_uint2(w[0], w[1]);
-          } else {
-#pragma unroll
-            for (int i = 0; i < VW; ++i)
-              if (n0 + i < N) yrow[n0 + i] = f32_to_bf16_bits(v[i] * gam);
-          }
-        }
-      }
+      wraw[PAR][f][0] = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 2048);
+      wraw[PAR][f][1] = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 2048 + 1024);
+      sd[PAR][f] = *reinterpret_cast<const uint32_t*>(sptr[f] + (int64_t)s * 128);
     }
+  };
+  // operands of step t of the stage held in LDS buffer `buf` / weight registers PAR
+  auto read_xf = [&](int buf, int t, int j, bf16x8_t (&out)[MFW]) __attribute__((always_inline)) {
+    out[j] = *reinterpret_cast<const bf16x8_t*>(lds + buf * XBYTES + (j * FM + lr) * XPITCH + h * 128 + t * 16);
+  };
+  // The empty volatile asm statements pin the conversion between the MFMAs of its slot: without them the
+  // (side-effect free) conversions drift to the start of the next step and serialise with the MFMAs.
+  auto make_wf = [&](auto par_c, int t, int f, bf16x8_t (&out)[NFW]) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_c)::value;
+    const u32x4_t v = wraw[PAR][f][t >> 2];
+    uint32_t raw = (t & 3) == 0 ? v.x : (t & 3) == 1 ? v.y : (t & 3) == 2 ? v.z : v.w;
+    asm volatile("" : "+v"(raw));
+    const uint32_t sbyte = (sd[PAR][f] >> (8 * (t >> 2))) >> (16 * h);  // MX block h*2 + t/4 of the stage
+    u32x4_t r = __builtin_bit_cast(u32x4_t, dequant8(raw, bits_f32((sbyte & 0xFFu) << 23)));
+    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+    out[f] = __builtin_bit_cast(bf16x8_t, r);
+  };
+
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+
+  // One K-stage.  NJ = row fragments with valid rows (compile-time so the MFMA list is straight-line code);
+  // only the 2*NJ activation pieces per thread that cover those fragments are staged.
+  auto stage = [&](auto nj_c, auto par_c, int c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    constexpr int PAR = decltype(par_c)::value;
+    using PARN = std::integral_constant<int, PAR ^ 1>;
+    constexpr int NM = NJ * NFW;
+    constexpr int NP = 2 * NJ;           // pieces to stage
+    constexpr int PPS = (NP + 3) / 4;    // per step, during steps 0..3
+    constexpr int NOPS = NJ + NFW + 2;   // NJ LDS reads, NFW conversions, two staging slots
+    static_for<0, 8>([&](auto t_c) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_c)::value;
+      constexpr int cur = t & 1, nxt = cur ^ 1;
+      auto op = [&](auto o_c) __attribute__((always_inline)) {
+        constexpr int o = decltype(o_c)::value;
+        if constexpr (t < 7) {
+          if constexpr (o < NJ) {
+            read_xf(PAR, t + 1, o, xf[nxt]);
+          } else if constexpr (o < NJ + NFW) {
+            make_wf(par_c, t + 1, o - NJ, wf[nxt]);
+          } else if constexpr (t < 4) {
+            // next stage's activations: registers -> LDS, then refill the registers for the stage after it
+            constexpr int half = o - NJ - NFW;
+            constexpr int j = t * PPS + half;
+            if constexpr (half < PPS && j < NP) {
+              store_x_piece(j, PAR ^ 1);
+              load_x_piece(j, c + 2);
+            }
+          }
+        } else {
+          if constexpr (o < NJ) {
+            read_xf(PAR ^ 1, 0, o, xf[nxt]);
+          } else if constexpr (o < NJ + NFW) {
+            make_wf(PARN{}, 0, o - NJ, wf[nxt]);
+          } else if constexpr (o == NJ + NFW + 1) {
+            load_w(par_c, c + 2);  // this stage's weight registers are free once step 7's operands exist
+          }
+        }
+      };
+      static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_c)::value;
+        constexpr int j = m / NFW, f = m % NFW;
+        acc[f][j] = FR::mma(wf[cur][f], xf[cur][j], acc[f][j]);
+        if constexpr (t == 7 && m == 0) {
+          // every wave has fetched its last operands of this buffer (during step 6) and written its share
+          // of the next one (steps 0..3)
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        }
+        // ops are dealt as evenly as possible: slot m runs ops [m*NOPS/NM, (m+1)*NOPS/NM)
+        static_for<(m * NOPS) / NM, ((m + 1) * NOPS) / NM>(op);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+
+  auto run = [&](auto nj_c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    constexpr int NP = 2 * NJ;
+    // prologue: stage 0 (and the loads of stage 1) without overlap
+#pragma unroll
+    for (int j = 0; j < NP; ++j) load_x_piece(j, 0);
+    load_w(P0{}, 0);
+    load_w(P1{}, 1);
+#pragma unroll
+    for (int j = 0; j < NP; ++j) store_x_piece(j, 0);
+#pragma unroll
+    for (int j = 0; j < NP; ++j) load_x_piece(j, 1);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) read_xf(0, 0, j, xf[0]);
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) make_wf(P0{}, 0, f, wf[0]);
+    for (int c = 0; c < nst; c += 2) {
+      stage(nj_c, P0{}, c);
+      if (c + 1 < nst) stage(nj_c, P1{}, c + 1);
+    }
+  };
+  if constexpr (MFW == 4) {
+    switch (nfrag_m) {
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      default: run(std::integral_constant<int, 4>{}); break;
+    }
+  } else {
+    if (nfrag_m == 1)
+      run(std::integral_constant<int, 1>{});
+    else
+      run(std::integral_constant<int, 2>{});
   }
+  gemm_epilogue<FM, 1, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, 0, lr, h);
+}
+
+template <int MFW>
+int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
+  constexpr int LDS_BYTES = 2 * MFW * 32 * (128 * 2 + 16);
+  GemmParams q = p;
+  q.grid_n = (int)cdiv(p.N, 256);
+  const int64_t grid = (int64_t)grid_m * q.grid_n;
+  if (grid <= 0) return TK_OK;
+  if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
+  auto launch = [&](auto kern) -> int32_t {
+    static bool attr_done = false;
+    if (!attr_done && LDS_BYTES > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
+      attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
+    return check_launch("moe_gemm_mxn_kernel");
+  };
+  if (swiglu) return launch(moe_gemm_mxn_kernel<MFW, true>);
+  return launch(moe_gemm_mxn_kernel<MFW, false>);
 }
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
@@ -635,7 +928,6 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->x_dtype != TK_BF16 && d->x_dtype != TK_E4M3) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16 or e4m3 (dtype %d)", d->x_dtype);
   if ((d->x_dtype == TK_E4M3) != (d->w_dtype == TK_E4M3)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: e4m3 activations go with e4m3 weights (x dtype %d, w dtype %d)", d->x_dtype, d->w_dtype);
   if (d->y_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16 (dtype %d)", d->y_dtype);
-  if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
   if (d->activation != TK_ACT_NONE && d->activation != TK_ACT_SWIGLU) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad activation %d", d->activation);
   if (d->activation == TK_ACT_SWIGLU && d->N % 2) return fail(TK_ERR_INVALID, "tk_moe_gemm: swiglu needs an even N");
   const int xe = d->x_dtype == TK_E4M3 ? 16 : 8;  // elements per 16 bytes
@@ -682,6 +974,18 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.grid_n = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
+  if (d->w_layout == TK_W_TILED) {
+    if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
+    if (d->block_m != 64 && d->block_m != 128) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout needs block_m 64 or 128 (got %d)", d->block_m);
+    if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w_mx_scale) & 3) || d->ws_stride_e % 4) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
+    const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
+    if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
+    p.w_stride_e = d->w_stride_e;
+    p.w_nst = (int32_t)nst;
+    return d->block_m == 64 ? launch_mxn<2>(p, d->grid_m, swiglu, st) : launch_mxn<4>(p, d->grid_m, swiglu, st);
+  }
+  if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);
+  if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
   if (d->w_dtype == TK_E2M1) {
     if (!d->w_mx_scale) return fail(TK_ERR_INVALID, "tk_moe_gemm: e2m1 weights need MX scales");
     if (d->ws_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: MX scales must be K-contiguous");

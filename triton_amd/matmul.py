@@ -29,6 +29,7 @@ from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_op
 from .numerics import InFlexData, OutFlexData
 from .specialize import FnSpecs
 from .tensor import FP4, RaggedTensorMetadata, Tensor, torch_dtype_to_dtype, wrap_torch_tensor
+from .tensor_details.layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
 from .tensor_details.layout_details.strided import StridedLayout
 
 MXFP_BLOCK_SIZE = 32
@@ -154,18 +155,21 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     b_scale = precision_config.b_mx_scale
     if not isinstance(b, Tensor):
         b = wrap_torch_tensor(b, dtype=FP4 if b.dtype == torch.uint8 else None)
-    if not isinstance(b.storage.layout, StridedLayout):
-        raise NotImplementedError("only strided weight layouts are supported")
+    tiled = isinstance(b.storage.layout, GFX950MXValueLayout)
+    if not tiled and not isinstance(b.storage.layout, StridedLayout):
+        raise NotImplementedError(f"weight layout {type(b.storage.layout).__name__} is not supported")
     if b_scale is not None and not isinstance(b_scale, Tensor):
         b_scale = wrap_torch_tensor(b_scale)
     if b_scale is not None:
-        if not isinstance(b_scale.storage.layout, StridedLayout):
-            raise NotImplementedError("only strided MX scale layouts are supported")
+        if tiled != isinstance(b_scale.storage.layout, GFX950MXScaleLayout):
+            raise NotImplementedError("tiled MXFP4 values go with tiled scales (convert both with convert_layout)")
+        if not tiled and not isinstance(b_scale.storage.layout, StridedLayout):
+            raise NotImplementedError(f"scale layout {type(b_scale.storage.layout).__name__} is not supported")
         assert b_scale.storage.data.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.storage.data.dtype}"
         assert precision_config.b_microblock_size is None or precision_config.b_microblock_size == MXFP_BLOCK_SIZE, \
             f"Unsupported microscale block size {precision_config.b_microblock_size}"
     w = b.storage.data
-    if w.ndim == 2:
+    if w.ndim == 2 and not tiled:
         w = w[None]
     K_W, N = b.shape[-2:]
     M = a.shape[-2] if gather_indx is None else gather_indx.shape[0]
@@ -215,7 +219,16 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         assert a_ts.numel() == a.shape[0], "a_mx_tensor_scale must hold one scale per row of a"
         d.x_row_scale = a_ts.data_ptr()
     keep = [a_ts]
-    if b.dtype == FP4:
+    if tiled:
+        assert b.dtype == FP4 and b_scale is not None, "tiled weights are MXFP4 and need precision_config.b_mx_scale"
+        ws = b_scale.storage.data
+        assert w.is_contiguous() and ws.is_contiguous() and ws.shape[0] == w.shape[0]
+        d.w_dtype = nt.TK_E2M1
+        d.w_layout = nt.TK_W_TILED
+        d.w_mx_scale = ws.data_ptr()
+        d.ws_stride_e = ws.stride(0)
+        keep.append(ws)
+    elif b.dtype == FP4:
         assert b_scale is not None, "mxfp4 weights need precision_config.b_mx_scale"
         assert w.dtype == torch.uint8
         if w.stride(-2) != 1:
@@ -233,7 +246,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         w = _k_contiguous(w)
         d.w_dtype = nt.TORCH_TO_TK.get(w.dtype, -1)
     d.w = w.data_ptr()
-    d.w_stride_e, d.w_stride_k, d.w_stride_n = w.stride()
+    if tiled:
+        d.w_stride_e = w.stride(0)
+    else:
+        d.w_stride_e, d.w_stride_k, d.w_stride_n = w.stride()
     keep.append(w)
     b_ts = precision_config.b_mx_tensor_scale
     if b_ts is not None:
@@ -265,6 +281,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         d.gammas_dtype = nt.TORCH_TO_TK[g.dtype]
         keep.append(g)
     block_m = opt_flags.block_m
+    if tiled and block_m < 64:
+        block_m = 64  # the tiled-layout kernel exists for 64- and 128-row blocks
     if is_ragged:
         md = a_ragged_metadata
         d.slice_sizes = md.slice_sizes.data_ptr()

@@ -1,21 +1,23 @@
 """Layouts accepted for matmul operands (mirrors `triton_kernels/tensor_details/layout.py`).
 
-Only the strided layout exists on gfx950 in this build; the default-layout helpers therefore return
-`StridedLayout(-2)` (K-major weights / scales), which is what the reference returns when no
-architecture-specific swizzle applies (layout.py:40,54).
+Two families exist on gfx950 in this build: the strided layout (what `downcast_to_mxfp` returns) and the
+pre-tiled MXFP4 pair `GFX950MXValueLayout` / `GFX950MXScaleLayout`, which the default-layout helpers return
+for weights whose MX axis is K, as the reference's helpers return its architecture-specific layouts
+(layout.py:26-54).  Both are accepted by `matmul`; the tiled pair is the fast path.
 """
 from .layout_details.base import Layout
+from .layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
 from .layout_details.strided import StridedLayout
 
-__all__ = ["Layout", "StridedLayout"]
+__all__ = ["Layout", "StridedLayout", "GFX950MXValueLayout", "GFX950MXScaleLayout"]
 
 
 def make_default_matmul_mxfp4_w_layout(mx_axis: int, **_unused):
-    return StridedLayout(-2)
+    return GFX950MXValueLayout() if mx_axis in (1, -2) else StridedLayout(-2)
 
 
 def make_default_matmul_mxfp4_w_scale_layout(mx_axis: int, num_warps: int = 8):
-    return StridedLayout(-2)
+    return GFX950MXScaleLayout() if mx_axis in (1, -2) else StridedLayout(-2)
 
 
 def make_default_matmul_mx_act_scale_layout(ragged_metadata=None):
