@@ -792,24 +792,34 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
   auto run = [&](auto nj_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
     constexpr int NP = 2 * NJ;
-    // prologue: stage 0 (and the loads of stage 1) without overlap
-#pragma unroll
-    for (int j = 0; j < NP; ++j) load_x_piece(j, 0);
+    // Prologue: stage 0 without overlap.  The order of the loads left in flight (weights of stage 0, activations
+    // of stage 1, weights of stage 1) is pinned to the order the steady state leaves them in at the top of an
+    // even stage: the compiler's wait counts at the loop header are the merge of both paths, and any mismatch
+    // makes every iteration wait for the loads it has just issued.
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0); });
+    __builtin_amdgcn_sched_barrier(0);
     load_w(P0{}, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0); });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1); });
+    __builtin_amdgcn_sched_barrier(0);
     load_w(P1{}, 1);
-#pragma unroll
-    for (int j = 0; j < NP; ++j) store_x_piece(j, 0);
-#pragma unroll
-    for (int j = 0; j < NP; ++j) load_x_piece(j, 1);
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) read_xf(0, 0, j, xf[0]);
-#pragma unroll
-    for (int f = 0; f < NFW; ++f) make_wf(P0{}, 0, f, wf[0]);
-    for (int c = 0; c < nst; c += 2) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { read_xf(0, 0, decltype(jc)::value, xf[0]); });
+    static_for<0, NFW>([&](auto fc) __attribute__((always_inline)) { make_wf(P0{}, 0, decltype(fc)::value, wf[0]); });
+    __builtin_amdgcn_sched_barrier(0);
+    // both stages of a pair always run inside the loop: a path that skips the odd stage and returns to the
+    // loop header would again make the header's wait counts cover the loads just issued
+    int c = 0;
+    for (; c + 1 < nst; c += 2) {
       stage(nj_c, P0{}, c);
-      if (c + 1 < nst) stage(nj_c, P1{}, c + 1);
+      stage(nj_c, P1{}, c + 1);
     }
+    if (c < nst) stage(nj_c, P0{}, c);
   };
   if constexpr (MFW == 4) {
     switch (nfrag_m) {
