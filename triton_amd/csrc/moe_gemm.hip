@@ -26,6 +26,9 @@
 namespace tk {
 namespace {
 
+template <int I>
+using template_int = std::integral_constant<int, I>;
+
 // f(integral_constant<int, I>) for I in [B, E), fully expanded at compile time
 template <int B, int E, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -327,10 +330,14 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
     const int live = p.block_offs[p.n_slices] * p.grid_n;
     if ((int)blockIdx.x >= live) return;
     const int pid = xcd_remap(blockIdx.x, live);
-    pid_n = pid % p.grid_n;
-    const int sched = p.block_sched[pid / p.grid_n];
-    expert = sched & 0xFFFF;
-    off_m = (sched >> 16) * BM;
+    // Tiles are ordered (expert, column tile, row block): the row blocks of one expert that share a column
+    // tile get consecutive ids, run at the same time on one XCD and stream the same weights through its L2.
+    expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
+    const int first = p.block_offs[expert];
+    const int nb = p.block_offs[expert + 1] - first;
+    const int local = pid - first * p.grid_n;
+    pid_n = local / nb;
+    off_m = (local - pid_n * nb) * BM;
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
@@ -615,10 +622,14 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 // by scheduling barriers, with the LDS reads and e2m1 -> bf16 conversions of step t+1, with the LDS writes of
 // the next stage's activations and the global loads of the stage after it.  One workgroup barrier per stage
 // sits in step 7, after every wave has fetched its last operands of the current LDS buffer.
-template <int MFW, bool SWIGLU>
-__global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
+//
+// G = row groups: with G = 2 the workgroup has eight waves; waves 0-3 own the even 32-row fragments of the tile
+// and waves 4-7 the odd ones (same columns), so every SIMD holds two waves whose MFMAs, conversions and memory
+// instructions overlap in hardware, while the weights are still fetched from L2 / HBM once per 64*MFW rows.
+template <int MFW, int G, bool SWIGLU>
+__global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams p) {
   typedef Frag<32> FR;
-  constexpr int FM = 32, NFW = 2, NT = 256, BM = MFW * 32, BN = 256, KC = 128;
+  constexpr int FM = 32, NFW = 2, NT = 256 * G, BM = MFW * 32 * G, BN = 256, KC = 128;
   constexpr int XPITCH = KC * 2 + 16;
   constexpr int XBYTES = BM * XPITCH;
   constexpr int XCH = BM * 16 / NT;  // 16-byte activation pieces per thread per stage (4 or 8)
@@ -629,10 +640,14 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
     const int live = p.block_offs[p.n_slices] * p.grid_n;
     if ((int)blockIdx.x >= live) return;
     const int pid = xcd_remap(blockIdx.x, live);
-    pid_n = pid % p.grid_n;
-    const int sched = p.block_sched[pid / p.grid_n];
-    expert = sched & 0xFFFF;
-    off_m = (sched >> 16) * BM;
+    // Tiles are ordered (expert, column tile, row block): the row blocks of one expert that share a column
+    // tile get consecutive ids, run at the same time on one XCD and stream the same weights through its L2.
+    expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
+    const int first = p.block_offs[expert];
+    const int nb = p.block_offs[expert + 1] - first;
+    const int local = pid - first * p.grid_n;
+    pid_n = local / nb;
+    off_m = (local - pid_n * nb) * BM;
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
@@ -647,7 +662,8 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
   const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int nw = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nw = wave & 3, grp = wave >> 2;  // column quarter, row group
   const int lr = lane & 31, h = lane >> 5;
   const int K = p.K, N = p.N;
   const int nst = p.w_nst;
@@ -657,13 +673,13 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
   const uint8_t* xptr[XCH];
 #pragma unroll
   for (int j = 0; j < XCH; ++j) {
-    const int r = (tid >> 4) + 16 * j;
+    const int r = (tid >> 4) + (NT / 16) * j;
     int row = off_m + r;
     row = row < eM ? row : eM - 1;
     const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
     xptr[j] = p.x + src * p.x_stride_m * 2;  // the k offset (incl. this thread's chunk) is added per stage
   }
-  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // piece j at xlds0 + j*16*XPITCH
+  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // piece j at xlds0 + j*(NT/16)*XPITCH
 
   // ---- weights: two column fragments of this wave ----
   const int nfr = (N + 31) >> 5;
@@ -685,22 +701,25 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
 #pragma unroll
       for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
 
-  u32x4_t xreg[XCH];  // native vectors: arrays of the HIP uint4 struct were left in scratch memory here
-  u32x4_t wraw[2][NFW][2];
-  uint32_t sd[2][NFW];
+  // activation staging registers, two stages deep: stage c writes X(c+1) from xreg[(c+1)&1] to LDS and refills it
+  // with X(c+3).  (Native vectors: arrays of the HIP uint4 struct were left in scratch memory here.)
+  u32x4_t xreg[2][XCH];
+  constexpr int WD = 4;  // weight register ring: stage c uses slot c % WD, loads run WD-1 stages ahead
+  u32x4_t wraw[WD][NFW][2];
+  uint32_t sd[WD][NFW];
   bf16x8_t xf[2][MFW];
   bf16x8_t wf[2][NFW];
 
   // Loads are unconditional (no divergent control flow inside the pipeline): rows past the tile's last
   // valid row re-read that row, k past K re-reads the row's last 8 values (the padded weights there are
   // zero), stages past the last one re-read the last stage.
-  auto load_x_piece = [&](int j, int s) __attribute__((always_inline)) {
+  auto load_x_piece = [&](int j, int s, int slot) __attribute__((always_inline)) {
     int k0 = s * KC + xc * 8;
     k0 = k0 < K - 8 ? k0 : K - 8;
-    xreg[j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0 * 2);
+    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0 * 2);
   };
-  auto store_x_piece = [&](int j, int buf) __attribute__((always_inline)) {
-    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 16 * XPITCH) = xreg[j];
+  auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * (NT / 16) * XPITCH) = xreg[slot][j];
   };
   auto load_w = [&](auto par_c, int s) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_c)::value;
@@ -714,7 +733,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
   };
   // operands of step t of the stage held in LDS buffer `buf` / weight registers PAR
   auto read_xf = [&](int buf, int t, int j, bf16x8_t (&out)[MFW]) __attribute__((always_inline)) {
-    out[j] = *reinterpret_cast<const bf16x8_t*>(lds + buf * XBYTES + (j * FM + lr) * XPITCH + h * 128 + t * 16);
+    out[j] = *reinterpret_cast<const bf16x8_t*>(lds + buf * XBYTES + ((j * G + grp) * FM + lr) * XPITCH + h * 128 + t * 16);
   };
   // The empty volatile asm statements pin the conversion between the MFMAs of its slot: without them the
   // (side-effect free) conversions drift to the start of the next step and serialise with the MFMAs.
@@ -729,17 +748,25 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
     out[f] = __builtin_bit_cast(bf16x8_t, r);
   };
 
-  using P0 = std::integral_constant<int, 0>;
-  using P1 = std::integral_constant<int, 1>;
+  template_int<0> S0;
+  template_int<1> S1;
+  template_int<2> S2;
+  template_int<3> S3;
 
   // One K-stage.  NJ = row fragments with valid rows (compile-time so the MFMA list is straight-line code);
-  // only the 2*NJ activation pieces per thread that cover those fragments are staged.
-  auto stage = [&](auto nj_c, auto par_c, int c) __attribute__((always_inline)) {
+  // only the 2*NJ activation pieces per thread that cover those fragments are staged.  WS = weight ring slot
+  // of this stage (= c % WD); the activation LDS buffer is WS & 1.
+  auto stage = [&](auto nj_c, auto gi_c, auto ws_c, int c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    constexpr int PAR = decltype(par_c)::value;
-    using PARN = std::integral_constant<int, PAR ^ 1>;
+    constexpr int WS = decltype(ws_c)::value;
+    constexpr int PAR = WS & 1;
+    using WSN = std::integral_constant<int, (WS + 1) % WD>;       // next stage's weights
+    using WSL = std::integral_constant<int, (WS + WD - 1) % WD>;  // slot to refill: stage c + WD - 1
+    constexpr int GI = decltype(gi_c)::value;  // this wave's row group
     constexpr int NM = NJ * NFW;
-    constexpr int NP = 2 * NJ;           // pieces to stage
+    // pieces to stage: a piece covers 16 rows (G = 1) or 32 rows (G = 2); with G = 2 the tile has 2*NJ - 1 or 2*NJ
+    // (group 0), 2*NJ or 2*NJ + 1 (group 1) fragments with valid rows, and the larger count is staged
+    constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
     constexpr int PPS = (NP + 3) / 4;    // per step, during steps 0..3
     constexpr int NOPS = NJ + NFW + 2;   // NJ LDS reads, NFW conversions, two staging slots
     static_for<0, 8>([&](auto t_c) __attribute__((always_inline)) {
@@ -751,26 +778,36 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
           if constexpr (o < NJ) {
             read_xf(PAR, t + 1, o, xf[nxt]);
           } else if constexpr (o < NJ + NFW) {
-            make_wf(par_c, t + 1, o - NJ, wf[nxt]);
+            make_wf(ws_c, t + 1, o - NJ, wf[nxt]);
           } else if constexpr (t < 4) {
             // next stage's activations: registers -> LDS, then refill the registers for the stage after it
             constexpr int half = o - NJ - NFW;
             constexpr int j = t * PPS + half;
             if constexpr (half < PPS && j < NP) {
-              store_x_piece(j, PAR ^ 1);
-              load_x_piece(j, c + 2);
+              store_x_piece(j, PAR ^ 1, PAR ^ 1);
+              load_x_piece(j, c + 3, PAR ^ 1);
             }
+          } else if constexpr (t == 4 && o == NJ + NFW) {
+            load_w(WSL{}, c + WD - 1);  // the slot of the previous stage is free
           }
         } else {
           if constexpr (o < NJ) {
             read_xf(PAR ^ 1, 0, o, xf[nxt]);
           } else if constexpr (o < NJ + NFW) {
-            make_wf(PARN{}, 0, o - NJ, wf[nxt]);
-          } else if constexpr (o == NJ + NFW + 1) {
-            load_w(par_c, c + 2);  // this stage's weight registers are free once step 7's operands exist
+            make_wf(WSN{}, 0, o - NJ, wf[nxt]);
           }
         }
       };
+      if constexpr (NM == 0) {
+        // a wave without valid rows still stages its share of the activations and joins the barriers
+        if constexpr (t == 7) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        }
+        static_for<0, NOPS>(op);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
         constexpr int m = decltype(m_c)::value;
         constexpr int j = m / NFW, f = m % NFW;
@@ -783,63 +820,91 @@ __global__ __launch_bounds__(256) void moe_gemm_mxn_kernel(const GemmParams p) {
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         }
         // ops are dealt as evenly as possible: slot m runs ops [m*NOPS/NM, (m+1)*NOPS/NM)
-        static_for<(m * NOPS) / NM, ((m + 1) * NOPS) / NM>(op);
+        static_for<(m * NOPS) / (NM ? NM : 1), ((m + 1) * NOPS) / (NM ? NM : 1)>(op);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
   };
 
-  auto run = [&](auto nj_c) __attribute__((always_inline)) {
+  auto run = [&](auto nj_c, auto gi_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    constexpr int NP = 2 * NJ;
-    // Prologue: stage 0 without overlap.  The order of the loads left in flight (weights of stage 0, activations
-    // of stage 1, weights of stage 1) is pinned to the order the steady state leaves them in at the top of an
-    // even stage: the compiler's wait counts at the loop header are the merge of both paths, and any mismatch
-    // makes every iteration wait for the loads it has just issued.
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0); });
+    constexpr int GI = decltype(gi_c)::value;
+    constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
+    // Prologue: stage 0 without overlap.  The order of the loads left in flight (activations, then weights, of
+    // stage 1, then of stage 2) is pinned to the order the steady state leaves them in at the top of a
+    // stage: the compiler's wait counts at the loop header are the merge of both paths, and any mismatch makes
+    // every iteration wait for the loads it has just issued.
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    load_w(P0{}, 0);
+    load_w(S0, 0);
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0); });
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1); });
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1); });
     __builtin_amdgcn_sched_barrier(0);
-    load_w(P1{}, 1);
+    load_w(S1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 2, 0); });
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(S2, 2);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { read_xf(0, 0, decltype(jc)::value, xf[0]); });
-    static_for<0, NFW>([&](auto fc) __attribute__((always_inline)) { make_wf(P0{}, 0, decltype(fc)::value, wf[0]); });
+    static_for<0, NFW>([&](auto fc) __attribute__((always_inline)) { make_wf(S0, 0, decltype(fc)::value, wf[0]); });
     __builtin_amdgcn_sched_barrier(0);
-    // both stages of a pair always run inside the loop: a path that skips the odd stage and returns to the
-    // loop header would again make the header's wait counts cover the loads just issued
+    // all stages of a group always run inside the loop: a path that skips some and returns to the loop header
+    // would again make the header's wait counts cover the loads just issued
     int c = 0;
-    for (; c + 1 < nst; c += 2) {
-      stage(nj_c, P0{}, c);
-      stage(nj_c, P1{}, c + 1);
+    for (; c + 3 < nst; c += 4) {
+      stage(nj_c, gi_c, S0, c);
+      stage(nj_c, gi_c, S1, c + 1);
+      stage(nj_c, gi_c, S2, c + 2);
+      stage(nj_c, gi_c, S3, c + 3);
     }
-    if (c < nst) stage(nj_c, P0{}, c);
+    if (c < nst) stage(nj_c, gi_c, S0, c);
+    if (c + 1 < nst) stage(nj_c, gi_c, S1, c + 1);
+    if (c + 2 < nst) stage(nj_c, gi_c, S2, c + 2);
   };
-  if constexpr (MFW == 4) {
-    switch (nfrag_m) {
-      case 1: run(std::integral_constant<int, 1>{}); break;
-      case 2: run(std::integral_constant<int, 2>{}); break;
-      case 3: run(std::integral_constant<int, 3>{}); break;
-      default: run(std::integral_constant<int, 4>{}); break;
+  // row fragments of this wave with valid rows: tile fragments grp, grp + G, ...
+  const int nj = (nfrag_m - grp + G - 1) / G;
+  auto dispatch = [&](auto gi_c) __attribute__((always_inline)) {
+    constexpr int GI = decltype(gi_c)::value;
+    if constexpr (GI == 1) {
+      if (nj == 0) {
+        run(template_int<0>{}, gi_c);
+        return;
+      }
     }
-  } else {
-    if (nfrag_m == 1)
-      run(std::integral_constant<int, 1>{});
+    if constexpr (MFW == 4) {
+      switch (nj) {
+        case 1: run(template_int<1>{}, gi_c); break;
+        case 2: run(template_int<2>{}, gi_c); break;
+        case 3: run(template_int<3>{}, gi_c); break;
+        default: run(template_int<4>{}, gi_c); break;
+      }
+    } else {
+      if (nj == 1)
+        run(template_int<1>{}, gi_c);
+      else
+        run(template_int<2>{}, gi_c);
+    }
+  };
+  if constexpr (G == 2) {
+    if (grp == 1)
+      dispatch(template_int<1>{});
     else
-      run(std::integral_constant<int, 2>{});
+      dispatch(template_int<0>{});
+  } else {
+    dispatch(template_int<0>{});
   }
-  gemm_epilogue<FM, 1, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, 0, lr, h);
+  gemm_epilogue<FM, G, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, grp, lr, h);
 }
 
-template <int MFW>
+template <int MFW, int G>
 int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
-  constexpr int LDS_BYTES = 2 * MFW * 32 * (128 * 2 + 16);
+  constexpr int LDS_BYTES = 2 * MFW * 32 * G * (128 * 2 + 16);
   GemmParams q = p;
   q.grid_n = (int)cdiv(p.N, 256);
   const int64_t grid = (int64_t)grid_m * q.grid_n;
@@ -852,11 +917,11 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
       if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
       attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256 * G), LDS_BYTES, st, q);
     return check_launch("moe_gemm_mxn_kernel");
   };
-  if (swiglu) return launch(moe_gemm_mxn_kernel<MFW, true>);
-  return launch(moe_gemm_mxn_kernel<MFW, false>);
+  if (swiglu) return launch(moe_gemm_mxn_kernel<MFW, G, true>);
+  return launch(moe_gemm_mxn_kernel<MFW, G, false>);
 }
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
@@ -992,7 +1057,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
-    return d->block_m == 64 ? launch_mxn<2>(p, d->grid_m, swiglu, st) : launch_mxn<4>(p, d->grid_m, swiglu, st);
+    return d->block_m == 64 ? launch_mxn<2, 1>(p, d->grid_m, swiglu, st) : launch_mxn<2, 2>(p, d->grid_m, swiglu, st);
   }
   if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);
   if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
