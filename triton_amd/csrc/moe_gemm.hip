@@ -19,6 +19,7 @@
 //     and is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 right before the MFMA;
 //   * the rows of a tile are dealt to the WM row-waves in interleaved 16-row fragments and fragments
 //     past the expert's last row are skipped, so a nearly empty row block costs almost no MFMA time.
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -101,13 +102,13 @@ __device__ inline bf16x8_t dequant8(uint32_t raw, float scale) {
   return r;
 }
 
-// s * (linear + 1), s = gate * sigmoid(alpha * gate); the reciprocal is the hardware approximation (1 ulp)
-__device__ inline float swiglu_f(float gate, float lin, float alpha, float limit, int has_limit) {
-  if (has_limit) {
-    gate = fminf(gate, limit);
-    lin = fminf(fmaxf(lin, -limit), limit);
-  }
-  const float s = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * gate));
+// s * (linear + 1), s = gate * sigmoid(alpha * gate).  `nalpha_log2e` = -alpha * log2(e); `limit` = +inf when the
+// activation has no limit.  v_med3_f32 clamps in one instruction; exp2 and the reciprocal are the hardware
+// approximations (1 ulp each).
+__device__ __forceinline__ float swiglu_f(float gate, float lin, float nalpha_log2e, float limit) {
+  gate = __builtin_amdgcn_fmed3f(gate, -INFINITY, limit);
+  lin = __builtin_amdgcn_fmed3f(lin, -limit, limit);
+  const float s = gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(nalpha_log2e * gate));
   return fmaf(s, lin, s);
 }
 
@@ -232,38 +233,47 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
   // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
   // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
   constexpr int VW = FM == 32 ? 8 : 4;
+  constexpr int NU = FR::NACC / VW;
+  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
+  const float limit = p.has_limit ? p.limit : INFINITY;
+  const bool fast = full_n && p.y_vec;  // every column of the tile exists and rows take vector stores
 #pragma unroll
   for (int j = 0; j < MFW; ++j) {
-    uint16_t* yrow = p.y + (ok[j] ? dst[j] : 0) * p.y_stride_m;
-    const float g = gam[j];
+    float v[NFW][NU][VW];
+    int n0[NFW][NU];
 #pragma unroll
-    for (int f = 0; f < NFW; ++f) {
+    for (int f = 0; f < NFW; ++f)
 #pragma unroll
-      for (int u = 0; u < FR::NACC / VW; ++u) {
-        float v[VW];
-        int n0;
+      for (int u = 0; u < NU; ++u) {
         if constexpr (FM == 32) {
           // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             uint32_t lo = f32_bits(acc[f][j][8 * u + i]), hi = f32_bits(acc[f][j][8 * u + 4 + i]);
             auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo's upper half <-> hi's lower half
-            v[i] = bits_f32(r[0]);
-            v[4 + i] = bits_f32(r[1]);
+            v[f][u][i] = bits_f32(r[0]);
+            v[f][u][4 + i] = bits_f32(r[1]);
           }
-          n0 = ncol0 + f * FM + 16 * u + 8 * h;
+          n0[f][u] = ncol0 + f * FM + 16 * u + 8 * h;
         } else {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = acc[f][j][4 * u + i];
-          n0 = ncol0 + f * FM + FR::n_of(4 * u, h);
+          for (int i = 0; i < 4; ++i) v[f][u][i] = acc[f][j][4 * u + i];
+          n0[f][u] = ncol0 + f * FM + FR::n_of(4 * u, h);
         }
-        if (!ok[j]) continue;
+      }
+    if (!ok[j]) continue;  // one divergent region per row fragment
+    uint16_t* yrow = p.y + dst[j] * p.y_stride_m;
+    const float g = gam[j];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
         if (SWIGLU) {
           float r[VW / 2];
 #pragma unroll
-          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[2 * i], v[2 * i + 1], p.alpha, p.limit, p.has_limit) * g;
-          const int o0 = n0 / 2;
-          if (o0 + VW / 2 <= NOUT && p.y_vec) {
+          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[f][u][2 * i], v[f][u][2 * i + 1], nalpha_log2e, limit) * g;
+          const int o0 = n0[f][u] / 2;
+          if (fast) {
             uint32_t w[VW / 4];
 #pragma unroll
             for (int i = 0; i < VW / 4; ++i) w[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
@@ -277,22 +287,21 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
               if (o0 + i < NOUT) yrow[o0 + i] = f32_to_bf16_bits(r[i]);
           }
         } else {
-          if (n0 + VW <= N && p.y_vec) {
+          if (fast) {
             uint32_t w[VW / 2];
 #pragma unroll
-            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[2 * i] * g, v[2 * i + 1] * g);
+            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[f][u][2 * i] * g, v[f][u][2 * i + 1] * g);
             if constexpr (VW == 8)
-              *reinterpret_cast<uint4*>(yrow + n0) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
+              *reinterpret_cast<uint4*>(yrow + n0[f][u]) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
             else
-              *reinterpret_cast<uint2*>(yrow + n0) = make_uint2(w[0], w[1]);
+              *reinterpret_cast<uint2*>(yrow + n0[f][u]) = make_uint2(w[0], w[1]);
           } else {
 #pragma unroll
             for (int i = 0; i < VW; ++i)
-              if (n0 + i < N) yrow[n0 + i] = f32_to_bf16_bits(v[i] * g);
+              if (n0[f][u] + i < N) yrow[n0[f][u] + i] = f32_to_bf16_bits(v[f][u][i] * g);
           }
         }
       }
-    }
   }
 }
 
@@ -626,10 +635,18 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 // G = row groups: with G = 2 the workgroup has eight waves; waves 0-3 own the even 32-row fragments of the tile
 // and waves 4-7 the odd ones (same columns), so every SIMD holds two waves whose MFMAs, conversions and memory
 // instructions overlap in hardware, while the weights are still fetched from L2 / HBM once per 64*MFW rows.
-template <int MFW, int G, bool SWIGLU>
+//
+// NFW = column fragments per wave (tile width 128 * NFW): the activation tile is fetched from L2 once per column
+// tile, so wider tiles cut the L2 -> L1 traffic, which is what bounds this kernel at prefill shapes.
+// WD / XD = depth of the weight register ring (2 or 4) / of the activation staging registers (1 or 2).
+// BLKM = rows of a row block in the ragged metadata (block_m).  A tile processes its block in passes of
+// BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 6 an expert of up to 192 rows is ONE tile (weights read
+// once, no nearly empty second tile) and only larger blocks take a second pass.
+template <int BLKM, int MFW, int NFW, int G, int WD, int XD, bool SWIGLU>
 __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams p) {
   typedef Frag<32> FR;
-  constexpr int FM = 32, NFW = 2, NT = 256 * G, BM = MFW * 32 * G, BN = 256, KC = 128;
+  constexpr int FM = 32, NT = 256 * G, BM = MFW * 32 * G, BN = 128 * NFW, KC = 128;
+  static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2), "ring depths");
   constexpr int XPITCH = KC * 2 + 16;
   constexpr int XBYTES = BM * XPITCH;
   constexpr int XCH = BM * 16 / NT;  // 16-byte activation pieces per thread per stage (4 or 8)
@@ -647,19 +664,17 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     const int nb = p.block_offs[expert + 1] - first;
     const int local = pid - first * p.grid_n;
     pid_n = local / nb;
-    off_m = (local - pid_n * nb) * BM;
+    off_m = (local - pid_n * nb) * BLKM;
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
     const int pid = xcd_remap(blockIdx.x, gridDim.x);
     pid_n = pid % p.grid_n;
     expert = 0;
-    off_m = (pid / p.grid_n) * BM;
+    off_m = (pid / p.grid_n) * BLKM;
     start_m = 0;
     eM = p.M;
   }
-  const int rows = (eM - off_m) < BM ? (eM - off_m) : BM;
-  const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -667,6 +682,12 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   const int lr = lane & 31, h = lane >> 5;
   const int K = p.K, N = p.N;
   const int nst = p.w_nst;
+  const int blk_off = off_m;
+  const int blk_rows = (eM - blk_off) < BLKM ? (eM - blk_off) : BLKM;
+  for (int pass_off = 0; pass_off < blk_rows; pass_off += BM) {
+  const int off_m = blk_off + pass_off;
+  const int rows = (blk_rows - pass_off) < BM ? (blk_rows - pass_off) : BM;
+  const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW*G)
 
   // ---- activation staging: this thread's 16-byte pieces (row r_j = tid/16 + 16 j, k-chunk c = tid%16) ----
   const int xc = tid & 15;
@@ -701,10 +722,10 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 #pragma unroll
       for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
 
-  // activation staging registers, two stages deep: stage c writes X(c+1) from xreg[(c+1)&1] to LDS and refills it
-  // with X(c+3).  (Native vectors: arrays of the HIP uint4 struct were left in scratch memory here.)
-  u32x4_t xreg[2][XCH];
-  constexpr int WD = 4;  // weight register ring: stage c uses slot c % WD, loads run WD-1 stages ahead
+  // activation staging registers, XD stages deep: stage c writes X(c+1) from slot (c+1) % XD to LDS and refills it
+  // with X(c+1+XD).  (Native vectors: arrays of the HIP uint4 struct were left in scratch memory here.)
+  u32x4_t xreg[XD][XCH];
+  // weight register ring: stage c uses slot c % WD, loads run WD-1 stages ahead
   u32x4_t wraw[WD][NFW][2];
   uint32_t sd[WD][NFW];
   bf16x8_t xf[2][MFW];
@@ -758,37 +779,40 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   // of this stage (= c % WD); the activation LDS buffer is WS & 1.
   auto stage = [&](auto nj_c, auto gi_c, auto ws_c, int c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    constexpr int WS = decltype(ws_c)::value;
-    constexpr int PAR = WS & 1;
-    using WSN = std::integral_constant<int, (WS + 1) % WD>;       // next stage's weights
-    using WSL = std::integral_constant<int, (WS + WD - 1) % WD>;  // slot to refill: stage c + WD - 1
+    constexpr int WS4 = decltype(ws_c)::value;  // c % 4
+    constexpr int PAR = WS4 & 1;
+    using WSC = template_int<WS4 % WD>;                // this stage's weights
+    using WSN = template_int<(WS4 + 1) % WD>;          // next stage's weights
+    using WSL = template_int<(WS4 + WD - 1) % WD>;     // slot to refill: stage c + WD - 1
+    constexpr int XS = (WS4 + 1) % XD;                 // activation register slot holding X(c+1)
+    constexpr int WLOAD_STEP = WD == 2 ? 0 : 4;        // the refilled slot was last read in step 6 of stage c-1
     constexpr int GI = decltype(gi_c)::value;  // this wave's row group
     constexpr int NM = NJ * NFW;
     // pieces to stage: a piece covers 16 rows (G = 1) or 32 rows (G = 2); with G = 2 the tile has 2*NJ - 1 or 2*NJ
     // (group 0), 2*NJ or 2*NJ + 1 (group 1) fragments with valid rows, and the larger count is staged
     constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
     constexpr int PPS = (NP + 3) / 4;    // per step, during steps 0..3
-    constexpr int NOPS = NJ + NFW + 2;   // NJ LDS reads, NFW conversions, two staging slots
+    constexpr int NOPS = NJ + NFW + 4;   // NJ LDS reads, NFW conversions, three staging slots, the weight loads
     static_for<0, 8>([&](auto t_c) __attribute__((always_inline)) {
       constexpr int t = decltype(t_c)::value;
       constexpr int cur = t & 1, nxt = cur ^ 1;
       auto op = [&](auto o_c) __attribute__((always_inline)) {
         constexpr int o = decltype(o_c)::value;
-        if constexpr (t < 7) {
+        if constexpr (o == NJ + NFW + 3) {
+          if constexpr (t == WLOAD_STEP) load_w(WSL{}, c + WD - 1);
+        } else if constexpr (t < 7) {
           if constexpr (o < NJ) {
             read_xf(PAR, t + 1, o, xf[nxt]);
           } else if constexpr (o < NJ + NFW) {
-            make_wf(ws_c, t + 1, o - NJ, wf[nxt]);
+            make_wf(WSC{}, t + 1, o - NJ, wf[nxt]);
           } else if constexpr (t < 4) {
-            // next stage's activations: registers -> LDS, then refill the registers for the stage after it
+            // next stage's activations: registers -> LDS, then refill the registers for a later stage
             constexpr int half = o - NJ - NFW;
             constexpr int j = t * PPS + half;
             if constexpr (half < PPS && j < NP) {
-              store_x_piece(j, PAR ^ 1, PAR ^ 1);
-              load_x_piece(j, c + 3, PAR ^ 1);
+              store_x_piece(j, PAR ^ 1, XS);
+              load_x_piece(j, c + 1 + XD, XS);
             }
-          } else if constexpr (t == 4 && o == NJ + NFW) {
-            load_w(WSL{}, c + WD - 1);  // the slot of the previous stage is free
           }
         } else {
           if constexpr (o < NJ) {
@@ -840,14 +864,20 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1); });
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1 % XD); });
     __builtin_amdgcn_sched_barrier(0);
-    load_w(S1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 2, 0); });
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(S2, 2);
-    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (WD == 4) {
+      load_w(S1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (XD == 2) {
+      static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 2, 0); });
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (WD == 4) {
+      load_w(S2, 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -877,19 +907,9 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
         return;
       }
     }
-    if constexpr (MFW == 4) {
-      switch (nj) {
-        case 1: run(template_int<1>{}, gi_c); break;
-        case 2: run(template_int<2>{}, gi_c); break;
-        case 3: run(template_int<3>{}, gi_c); break;
-        default: run(template_int<4>{}, gi_c); break;
-      }
-    } else {
-      if (nj == 1)
-        run(template_int<1>{}, gi_c);
-      else
-        run(template_int<2>{}, gi_c);
-    }
+    static_for<1, MFW + 1>([&](auto n_c) __attribute__((always_inline)) {
+      if (nj == decltype(n_c)::value) run(n_c, gi_c);
+    });
   };
   if constexpr (G == 2) {
     if (grp == 1)
@@ -899,14 +919,15 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   } else {
     dispatch(template_int<0>{});
   }
-  gemm_epilogue<FM, G, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, grp, lr, h);
+  gemm_epilogue<FM, G, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, blk_off + blk_rows, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, grp, lr, h);
+  }  // passes
 }
 
-template <int MFW, int G>
+template <int BLKM, int MFW, int NFW, int G, int WD, int XD>
 int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
   constexpr int LDS_BYTES = 2 * MFW * 32 * G * (128 * 2 + 16);
   GemmParams q = p;
-  q.grid_n = (int)cdiv(p.N, 256);
+  q.grid_n = (int)cdiv(p.N, 128 * NFW);
   const int64_t grid = (int64_t)grid_m * q.grid_n;
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
@@ -920,8 +941,8 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256 * G), LDS_BYTES, st, q);
     return check_launch("moe_gemm_mxn_kernel");
   };
-  if (swiglu) return launch(moe_gemm_mxn_kernel<MFW, G, true>);
-  return launch(moe_gemm_mxn_kernel<MFW, G, false>);
+  if (swiglu) return launch(moe_gemm_mxn_kernel<BLKM, MFW, NFW, G, WD, XD, true>);
+  return launch(moe_gemm_mxn_kernel<BLKM, MFW, NFW, G, WD, XD, false>);
 }
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
@@ -1051,13 +1072,21 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
-    if (d->block_m != 64 && d->block_m != 128) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout needs block_m 64 or 128 (got %d)", d->block_m);
+    if (d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout needs block_m 64, 128 or 256 (got %d)", d->block_m);
     if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w_mx_scale) & 3) || d->ws_stride_e % 4) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
     const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
-    return d->block_m == 64 ? launch_mxn<2, 1>(p, d->grid_m, swiglu, st) : launch_mxn<2, 2>(p, d->grid_m, swiglu, st);
+    {
+      const char* v = getenv("TK_MXN");  // experiment switch
+      const int variant = v ? atoi(v) : 0;
+      if (d->block_m == 64) return launch_mxn<64, 2, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
+      if (d->block_m == 256) return launch_mxn<256, 6, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
+      if (variant == 1) return launch_mxn<128, 2, 2, 2, 4, 2>(p, d->grid_m, swiglu, st);
+      if (variant == 4) return launch_mxn<128, 4, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
+      return launch_mxn<128, 4, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
+    }
   }
   if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);
   if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
