@@ -58,6 +58,18 @@ def make_moe_weights(E, d_model, d_ff2, seed, device, n_copies=1):
     return out
 
 
+def to_matmul_layout(weights):
+    """Expert weights in the layouts `matmul` prefers on this GPU, converted once as a model loader would (the
+    reference's benchmark does the same with its `make_default_matmul_mxfp4_w_layout`, bench/bench_mlp.py:40-58)."""
+    from triton_kernels.tensor import FP4, convert_layout, wrap_torch_tensor
+    from triton_kernels.tensor_details.layout import make_default_matmul_mxfp4_w_layout, make_default_matmul_mxfp4_w_scale_layout
+    out = dict(weights)
+    for name in ("w1", "w2"):
+        out[name] = convert_layout(wrap_torch_tensor(weights[name], dtype=FP4), make_default_matmul_mxfp4_w_layout(mx_axis=1))
+        out[name + "s"] = convert_layout(wrap_torch_tensor(weights[name + "s"]), make_default_matmul_mxfp4_w_scale_layout(mx_axis=1))
+    return out
+
+
 class MoeLayer:
     """The hot path composed from the drop-in API (triton_kernels names)."""
 
@@ -246,7 +258,7 @@ def main():
     g = torch.Generator().manual_seed(2)
     x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
     logits = torch.randn((T, E), generator=g).to(device)
-    weights = make_moe_weights(E, d, f2, seed=2, device=device)[0]
+    weights = to_matmul_layout(make_moe_weights(E, d, f2, seed=2, device=device)[0])
     layer = MoeLayer(weights, k)
     if args.calibrate_copy:
         calibration_copy(device)

@@ -19,7 +19,6 @@
 //     and is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 right before the MFMA;
 //   * the rows of a tile are dealt to the WM row-waves in interleaved 16-row fragments and fragments
 //     past the expert's last row are skipped, so a nearly empty row block costs almost no MFMA time.
-#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -78,6 +77,7 @@ struct GemmParams {
   int32_t y_vec;     // output rows allow 16-byte vector stores
   int32_t bias_vec;  // bias rows allow 16-byte vector loads
   int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
+  int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
 };
 
 __device__ inline int xcd_remap(int pid, int total) {
@@ -652,11 +652,23 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   constexpr int XCH = BM * 16 / NT;  // 16-byte activation pieces per thread per stage (4 or 8)
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nw = wave & 3, grp = wave >> 2;  // column quarter, row group
+  const int lr = lane & 31, h = lane >> 5;
+  const int K = p.K, N = p.N;
+  const int nst = p.w_nst;
+  // Persistent workgroups: the grid is a few workgroups per CU and each walks over tiles round by round, so
+  // no CU waits for the dispatcher between tiles.  A round is gridDim.x consecutive tile ids; inside a round
+  // the ids are dealt so that each XCD (which receives every 8th workgroup) works on a contiguous run.
+  const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
+  for (int round0 = 0; round0 < live; round0 += (int)gridDim.x) {
+  const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
+  if ((int)blockIdx.x >= in_round) break;
+  const int pid = round0 + xcd_remap(blockIdx.x, in_round);
   int expert, off_m, start_m, eM, pid_n;
   if (p.slice_sizes) {
-    const int live = p.block_offs[p.n_slices] * p.grid_n;
-    if ((int)blockIdx.x >= live) return;
-    const int pid = xcd_remap(blockIdx.x, live);
     // Tiles are ordered (expert, column tile, row block): the row blocks of one expert that share a column
     // tile get consecutive ids, run at the same time on one XCD and stream the same weights through its L2.
     expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
@@ -668,20 +680,12 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
-    const int pid = xcd_remap(blockIdx.x, gridDim.x);
     pid_n = pid % p.grid_n;
     expert = 0;
     off_m = (pid / p.grid_n) * BLKM;
     start_m = 0;
     eM = p.M;
   }
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nw = wave & 3, grp = wave >> 2;  // column quarter, row group
-  const int lr = lane & 31, h = lane >> 5;
-  const int K = p.K, N = p.N;
-  const int nst = p.w_nst;
   const int blk_off = off_m;
   const int blk_rows = (eM - blk_off) < BLKM ? (eM - blk_off) : BLKM;
   for (int pass_off = 0; pass_off < blk_rows; pass_off += BM) {
@@ -921,6 +925,20 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   }
   gemm_epilogue<FM, G, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, blk_off + blk_rows, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, grp, lr, h);
   }  // passes
+  }  // rounds
+}
+
+// compute units of the current device (cached per device id)
+inline int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
 }
 
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD>
@@ -928,9 +946,14 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   constexpr int LDS_BYTES = 2 * MFW * 32 * G * (128 * 2 + 16);
   GemmParams q = p;
   q.grid_n = (int)cdiv(p.N, 128 * NFW);
-  const int64_t grid = (int64_t)grid_m * q.grid_n;
+  int64_t grid = (int64_t)grid_m * q.grid_n;
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
+  q.total_tiles = (int32_t)grid;
+  // persistent grid: as many workgroups as fit on the device at once (LDS decides how many share a CU)
+  const int per_cu = LDS_BYTES > 80 * 1024 ? 1 : 2;
+  const int64_t resident = (int64_t)device_cu_count() * per_cu;
+  if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
     static bool attr_done = false;
     if (!attr_done && LDS_BYTES > 64 * 1024) {
@@ -1078,15 +1101,10 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
-    {
-      const char* v = getenv("TK_MXN");  // experiment switch
-      const int variant = v ? atoi(v) : 0;
-      if (d->block_m == 64) return launch_mxn<64, 2, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
-      if (d->block_m == 256) return launch_mxn<256, 6, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
-      if (variant == 1) return launch_mxn<128, 2, 2, 2, 4, 2>(p, d->grid_m, swiglu, st);
-      if (variant == 4) return launch_mxn<128, 4, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
-      return launch_mxn<128, 4, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
-    }
+    //                                  BLKM MFW NFW G WD XD
+    if (d->block_m == 64) return launch_mxn<64, 2, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
+    if (d->block_m == 256) return launch_mxn<256, 6, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
+    return launch_mxn<128, 4, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
   }
   if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);
   if (d->w_stride_k != 1) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weights must be K-contiguous (stride_k == 1)");
