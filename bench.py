@@ -184,7 +184,7 @@ def bench_decode(device, steps, warmup):
     weight copies are rotated so no step finds its weights in the last-level cache.  Every replay's output is
     checked against the eager result before timing."""
     E, k, d, f2 = 128, 4, 2880, 5760
-    copies = make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)
+    copies = [to_matmul_layout(w) for w in make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)]
     per_expert = d * f2 // 2 + d * f2 // 32 + (f2 // 2) * d // 2 + (f2 // 2) * d // 32
     res = {}
     g = torch.Generator().manual_seed(3)

@@ -69,7 +69,7 @@ CASES = [
 
 
 @pytest.mark.parametrize("m, n, k, mode, wkind", CASES)
-@pytest.mark.parametrize("block_m", [16, 64, 128, 256])
+@pytest.mark.parametrize("block_m", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("do_gather, do_scatter", [(False, False), (True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("do_gamma", [False, True])
 def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatter, do_gamma):

@@ -928,6 +928,162 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   }  // rounds
 }
 
+// ------------------------------------------------------------------------------------------------
+// MXFP4 weights in the tile-native layout, decode shapes (block_m 16 / 32): a pure weight stream
+// ------------------------------------------------------------------------------------------------
+// A few rows per expert: the kernel is bound by reading each active expert's weights once.  Every wave works
+// alone (no LDS, no barrier): it owns one 32-column weight fragment of one row block, streams the fragment's
+// K-stages through a six-deep register ring (12 KiB in flight per wave, up to sixteen waves per CU), reads its
+// rows' activations straight from L2 (each lane 64 contiguous bytes per stage), and issues 16x16x32 MFMAs
+// transposed like the prefill kernel (lane = column, 4 k-groups).  Within a stage lane group kg owns
+// k in [kg*32, kg*32 + 32): exactly one MX block and one 16-byte piece of the tiled layout.
+template <int MR, bool SWIGLU>
+__global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
+  typedef Frag<16> FR;
+  constexpr int WDD = 6, XDD = 3;  // ring depths (stages) of the weight / activation registers
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, kg = lane >> 4;
+  const int K = p.K, N = p.N;
+  const int nst = p.w_nst;
+  const int nfr = (N + 31) >> 5;
+
+  int expert, off_m, start_m, eM, pid_n;
+  if (p.slice_sizes) {
+    const int live = p.block_offs[p.n_slices] * p.grid_n;
+    if ((int)blockIdx.x >= live) return;
+    const int pid = blockIdx.x;
+    pid_n = pid % p.grid_n;
+    const int sched = p.block_sched[pid / p.grid_n];
+    expert = sched & 0xFFFF;
+    off_m = (sched >> 16) * (MR * 16);
+    start_m = p.slice_offs[expert];
+    eM = p.slice_sizes[expert];
+  } else {
+    const int pid = blockIdx.x;
+    pid_n = pid % p.grid_n;
+    expert = 0;
+    off_m = (pid / p.grid_n) * (MR * 16);
+    start_m = 0;
+    eM = p.M;
+  }
+  int F = pid_n * 4 + wave;  // this wave's 32-column fragment
+  const bool live_wave = F < nfr;
+  F = live_wave ? F : nfr - 1;
+  const int rows = (eM - off_m) < MR * 16 ? (eM - off_m) : MR * 16;
+  const int nj = (rows + 15) >> 4;  // row fragments with valid rows (1..MR)
+
+  // weights: sub-fragment g holds columns F*32 + g*16 + lr; this lane's piece of a stage is k-block kg
+  const uint8_t* wbase = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 2048 + (kg & 1) * 1024 + ((kg >> 1) * 32 + lr) * 16;
+  const uint8_t* sbase = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)F * nst * 128 + lr * 4;
+  // activations: row j*16 + lr, 64 bytes per stage at k offset kg*32
+  const uint8_t* xptr[MR];
+#pragma unroll
+  for (int j = 0; j < MR; ++j) {
+    int row = off_m + j * 16 + lr;
+    row = row < eM ? row : eM - 1;
+    const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
+    xptr[j] = p.x + src * p.x_stride_m * 2;
+  }
+
+  typename FR::acc_t acc[2][MR];
+#pragma unroll
+  for (int g = 0; g < 2; ++g)
+#pragma unroll
+    for (int j = 0; j < MR; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[g][j][i] = 0.f;
+
+  u32x4_t wr[WDD][2];
+  uint32_t sr[WDD][2];
+  u32x4_t xr[XDD][MR][4];
+
+  auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
+    constexpr int SL = decltype(slot_c)::value;
+    s = s < nst ? s : nst - 1;
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      wr[SL][g] = *reinterpret_cast<const u32x4_t*>(wbase + (int64_t)s * 2048 + g * 256);
+      sr[SL][g] = *reinterpret_cast<const uint32_t*>(sbase + (int64_t)s * 128 + g * 64);
+    }
+  };
+  auto load_x = [&](auto slot_c, int s) __attribute__((always_inline)) {
+    constexpr int SL = decltype(slot_c)::value;
+#pragma unroll
+    for (int j = 0; j < MR; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        int k0 = s * 128 + kg * 32 + t * 8;
+        k0 = k0 < K - 8 ? k0 : K - 8;  // past K the padded weights are zero; any finite activation will do
+        xr[SL][j][t] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0 * 2);
+      }
+  };
+  auto compute = [&](auto wslot_c, auto xslot_c) __attribute__((always_inline)) {
+    constexpr int WS = decltype(wslot_c)::value;
+    constexpr int XS = decltype(xslot_c)::value;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      bf16x8_t wf[2];
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const u32x4_t v = wr[WS][g];
+        const uint32_t raw = t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
+        wf[g] = dequant8(raw, bits_f32(((sr[WS][g] >> (8 * kg)) & 0xFFu) << 23));
+      }
+#pragma unroll
+      for (int j = 0; j < MR; ++j) {
+        if (j < nj) {
+          const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xr[XS][j][t]);
+#pragma unroll
+          for (int g = 0; g < 2; ++g) acc[g][j] = FR::mma(wf[g], xf, acc[g][j]);
+        }
+      }
+    }
+  };
+
+  if (live_wave) {
+    // prologue: fill the rings in the order the steady state leaves them (weights run WDD-1 stages ahead,
+    // activations XDD-1)
+    static_for<0, WDD - 1>([&](auto c_c) __attribute__((always_inline)) {
+      constexpr int c = decltype(c_c)::value;
+      load_w(c_c, c);
+      if constexpr (c < XDD - 1) load_x(c_c, c);
+    });
+    int c = 0;
+    for (; c + WDD - 1 < nst; c += WDD) {
+      static_for<0, WDD>([&](auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        load_w(template_int<(i + WDD - 1) % WDD>{}, c + i + WDD - 1);
+        load_x(template_int<(i + XDD - 1) % XDD>{}, c + i + XDD - 1);
+        compute(i_c, template_int<i % XDD>{});
+      });
+    }
+    static_for<0, WDD - 1>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if (c + i < nst) {
+        load_x(template_int<(i + XDD - 1) % XDD>{}, c + i + XDD - 1);
+        compute(i_c, template_int<i % XDD>{});
+      }
+    });
+    gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc, expert, off_m, start_m, eM, F * 32, F * 32 + 32 <= N, 0, lr, kg);
+  }
+}
+
+template <int MR>
+int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
+  GemmParams q = p;
+  q.grid_n = (int)cdiv(cdiv(p.N, 32), 4);
+  const int64_t grid = (int64_t)grid_m * q.grid_n;
+  if (grid <= 0) return TK_OK;
+  if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
+  if (swiglu)
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, true>), dim3((unsigned)grid), dim3(256), 0, st, q);
+  else
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, false>), dim3((unsigned)grid), dim3(256), 0, st, q);
+  return check_launch("moe_gemm_mxd_kernel");
+}
+
 // compute units of the current device (cached per device id)
 inline int device_cu_count() {
   static int cached[64] = {0};
@@ -1095,13 +1251,15 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
-    if (d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout needs block_m 64, 128 or 256 (got %d)", d->block_m);
+    if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);
     if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w_mx_scale) & 3) || d->ws_stride_e % 4) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
     const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
     //                                  BLKM MFW NFW G WD XD
+    if (d->block_m == 16) return launch_mxd<1>(p, d->grid_m, swiglu, st);
+    if (d->block_m == 32) return launch_mxd<2>(p, d->grid_m, swiglu, st);
     if (d->block_m == 64) return launch_mxn<64, 2, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
     if (d->block_m == 256) return launch_mxn<256, 6, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
     return launch_mxn<128, 4, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
