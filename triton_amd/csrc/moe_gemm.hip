@@ -940,7 +940,8 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 template <int MR, bool SWIGLU>
 __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   typedef Frag<16> FR;
-  constexpr int WDD = 6, XDD = 3;  // ring depths (stages) of the weight / activation registers
+  constexpr int WDD = 4, XDD = 2;  // ring depths (stages) of the weight / activation registers
+  __shared__ float red[3][2 * MR * 4][64];  // K-split partial sums of waves 1..3
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -949,30 +950,38 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   const int nst = p.w_nst;
   const int nfr = (N + 31) >> 5;
 
-  int expert, off_m, start_m, eM, pid_n;
+  // K-split: when few tiles are live (a handful of active experts), 2 or 4 waves share a fragment and take
+  // every 2nd / 4th K-stage each, so that enough loads are in flight to cover the HBM latency.  The factor is
+  // derived on the device from the live block count (the host never reads it) and is uniform over the grid;
+  // the grid is launched for the largest factor and the surplus workgroups leave at once.
+  const int nblk = p.slice_sizes ? p.block_offs[p.n_slices] : p.total_tiles;
+  const int frag_tiles = nblk * nfr;  // (row block, fragment) pairs = waves at split 1
+  const int ksplit = frag_tiles <= 1024 ? 4 : (frag_tiles <= 2048 ? 2 : 1);
+  const int fpw = 4 / ksplit;                        // fragments per workgroup
+  const int grid_n = (nfr + fpw - 1) / fpw;          // workgroups per row block
+  if ((int)blockIdx.x >= nblk * grid_n) return;
+  const int pid_n = blockIdx.x % grid_n, pid_m = blockIdx.x / grid_n;
+  const int kslice = wave % ksplit;
+  int expert, off_m, start_m, eM;
   if (p.slice_sizes) {
-    const int live = p.block_offs[p.n_slices] * p.grid_n;
-    if ((int)blockIdx.x >= live) return;
-    const int pid = blockIdx.x;
-    pid_n = pid % p.grid_n;
-    const int sched = p.block_sched[pid / p.grid_n];
+    const int sched = p.block_sched[pid_m];
     expert = sched & 0xFFFF;
     off_m = (sched >> 16) * (MR * 16);
     start_m = p.slice_offs[expert];
     eM = p.slice_sizes[expert];
   } else {
-    const int pid = blockIdx.x;
-    pid_n = pid % p.grid_n;
     expert = 0;
-    off_m = (pid / p.grid_n) * (MR * 16);
+    off_m = pid_m * (MR * 16);
     start_m = 0;
     eM = p.M;
   }
-  int F = pid_n * 4 + wave;  // this wave's 32-column fragment
+  int F = pid_n * fpw + wave / ksplit;  // this wave's 32-column fragment
   const bool live_wave = F < nfr;
   F = live_wave ? F : nfr - 1;
   const int rows = (eM - off_m) < MR * 16 ? (eM - off_m) : MR * 16;
   const int nj = (rows + 15) >> 4;  // row fragments with valid rows (1..MR)
+  // this wave's stages: kslice, kslice + ksplit, ...
+  const int my_nst = (nst - kslice + ksplit - 1) / ksplit;
 
   // weights: sub-fragment g holds columns F*32 + g*16 + lr; this lane's piece of a stage is k-block kg
   const uint8_t* wbase = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 2048 + (kg & 1) * 1024 + ((kg >> 1) * 32 + lr) * 16;
@@ -999,8 +1008,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   uint32_t sr[WDD][2];
   u32x4_t xr[XDD][MR][4];
 
-  auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
+  // `i` counts this wave's own stages; the global stage is kslice + i*ksplit (clamped: surplus loads re-read
+  // the last stage and are never used)
+  auto load_w = [&](auto slot_c, int i) __attribute__((always_inline)) {
     constexpr int SL = decltype(slot_c)::value;
+    int s = kslice + i * ksplit;
     s = s < nst ? s : nst - 1;
 #pragma unroll
     for (int g = 0; g < 2; ++g) {
@@ -1008,8 +1020,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
       sr[SL][g] = *reinterpret_cast<const uint32_t*>(sbase + (int64_t)s * 128 + g * 64);
     }
   };
-  auto load_x = [&](auto slot_c, int s) __attribute__((always_inline)) {
+  auto load_x = [&](auto slot_c, int i) __attribute__((always_inline)) {
     constexpr int SL = decltype(slot_c)::value;
+    const int s = kslice + i * ksplit;
 #pragma unroll
     for (int j = 0; j < MR; ++j)
 #pragma unroll
@@ -1051,7 +1064,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
       if constexpr (c < XDD - 1) load_x(c_c, c);
     });
     int c = 0;
-    for (; c + WDD - 1 < nst; c += WDD) {
+    for (; c + WDD - 1 < my_nst; c += WDD) {
       static_for<0, WDD>([&](auto i_c) __attribute__((always_inline)) {
         constexpr int i = decltype(i_c)::value;
         load_w(template_int<(i + WDD - 1) % WDD>{}, c + i + WDD - 1);
@@ -1061,20 +1074,42 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     }
     static_for<0, WDD - 1>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value;
-      if (c + i < nst) {
+      if (c + i < my_nst) {
         load_x(template_int<(i + XDD - 1) % XDD>{}, c + i + XDD - 1);
         compute(i_c, template_int<i % XDD>{});
       }
     });
-    gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc, expert, off_m, start_m, eM, F * 32, F * 32 + 32 <= N, 0, lr, kg);
   }
+  if (ksplit > 1) {
+    // sum the K-slices of a fragment in the wave with kslice 0 (through LDS), which then runs the epilogue
+    if (kslice != 0) {
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int j = 0; j < MR; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) red[wave - 1][(g * MR + j) * 4 + i][lane] = acc[g][j][i];
+    }
+    __syncthreads();
+    if (kslice != 0) return;
+    for (int o = 1; o < ksplit; ++o)
+#pragma unroll
+      for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int j = 0; j < MR; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[g][j][i] += red[wave + o - 1][(g * MR + j) * 4 + i][lane];
+  }
+  if (live_wave)
+    gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc, expert, off_m, start_m, eM, F * 32, F * 32 + 32 <= N, 0, lr, kg);
 }
 
 template <int MR>
 int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
   GemmParams q = p;
-  q.grid_n = (int)cdiv(cdiv(p.N, 32), 4);
-  const int64_t grid = (int64_t)grid_m * q.grid_n;
+  q.total_tiles = grid_m;  // row blocks in the non-ragged case
+  // sized for a K-split of 4 (one fragment per workgroup); with a smaller split the surplus leaves at once
+  const int64_t grid = (int64_t)grid_m * cdiv(p.N, 32);
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   if (swiglu)

@@ -366,6 +366,152 @@ __global__ __launch_bounds__(kScanThreads) void ragged_metadata_kernel(const int
   ragged_metadata(slice_sizes, E, nullptr, r, true);
 }
 
+// ---- whole routing pass in ONE workgroup (small batches) ------------------------------------------
+// For T*k <= kSmallEntries the three phases run back to back in a single 1024-thread workgroup: the waves take
+// rows round-robin for the top-k, the selected expert ids stay in LDS, the histogram is built with LDS atomics,
+// an entry's stable rank inside its expert is a count over the earlier entries (at most kSmallEntries LDS
+// reads, all lanes reading the same address), and the ragged metadata follows.  One launch instead of three:
+// at decode batch sizes the pass is pure launch latency.
+constexpr int kSmallEntries = 1024;
+
+struct SmallParams {
+  TopkParams t;
+  int32_t* col_sum;
+  int32_t* col_offs;  // [E+1] scratch
+  int32_t* col_sorted;
+  int32_t* row_sorted;
+  int32_t* gather_out;
+  void* gammas_out;
+  int32_t vals_bytes;
+  int32_t want_ragged;
+  RaggedOut r;
+};
+
+template <int DT, int EPL>
+__global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallParams q) {
+  __shared__ int32_t eid_s[kSmallEntries];
+  __shared__ uint32_t val_s[kSmallEntries];
+  __shared__ int32_t hist_s[kMaxExperts];
+  __shared__ uint32_t words_s[kScanWaves][EPL * 2];
+  const TopkParams& p = q.t;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int E = p.E, k = p.k, T = p.T;
+  const int n_rows = p.n_rows_ptr ? *p.n_rows_ptr : p.n_rows_imm;
+  const int words = (E + 31) / 32;
+  const int R = T * k;
+  for (int e = threadIdx.x; e < E; e += kScanThreads) hist_s[e] = 0;
+  for (int f = threadIdx.x; f < R; f += kScanThreads) eid_s[f] = -1;
+  __syncthreads();
+  // ---- phase 1: top-k per row (wave w takes rows w, w + 16, ...) ----
+  for (int row = wave; row < T && row < n_rows; row += kScanWaves) {
+    float myval = 0.f;
+    int myidx = -1;
+    if (p.use_provided_indx) {
+      if (lane < k) {
+        myidx = p.indx[(int64_t)row * k + lane];
+        if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
+      }
+    } else {
+      unsigned long long key[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        key[i] = 0ull;
+        if (e < E) {
+          const float v = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e);
+          key[i] = ((unsigned long long)ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e);
+        }
+      }
+      for (int j = 0; j < k; ++j) {
+        unsigned long long best = key[0];
+#pragma unroll
+        for (int i = 1; i < EPL; ++i) best = key[i] > best ? key[i] : best;
+        best = wave_max_u64(best);
+#pragma unroll
+        for (int i = 0; i < EPL; ++i)
+          if (key[i] == best) key[i] = 0ull;
+        if (lane == j) {
+          myval = key_to_float((uint32_t)(best >> 32));
+          myidx = (int)(~(uint32_t)best);
+        }
+      }
+    }
+    float outv = myval;
+    if (p.apply_softmax) {
+      float vmax;
+      if (p.use_provided_indx) {
+        float m = lane < k ? myval : -INFINITY;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+        vmax = m;
+      } else {
+        vmax = __shfl(myval, 0);
+      }
+      const float z = lane < k ? expf(myval - vmax) : 0.f;
+      const float sum = wave_sum_f32(z);
+      outv = z / sum;
+    }
+    const bool live = lane < k && myidx >= 0 && myidx < E;
+    if (lane < k) {
+      if (p.vals) store_val<DT>(p.vals, (int64_t)row * k + lane, outv);
+      if (!p.use_provided_indx) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
+      eid_s[row * k + lane] = live ? myidx : -1;
+      // the gate value as it is stored (bits of the logits dtype)
+      uint32_t bits;
+      if (DT == TK_F32)
+        bits = f32_bits(outv);
+      else if (DT == TK_BF16)
+        bits = f32_to_bf16_bits(outv);
+      else
+        bits = f32_to_f16_bits(outv);
+      val_s[row * k + lane] = bits;
+    }
+    if (live) atomicAdd(&hist_s[myidx], 1);
+    if (p.bitmatrix) {
+      for (int w = lane; w < words; w += 64) words_s[wave][w] = 0u;
+      wave_sync();
+      if (live) atomicOr(&words_s[wave][myidx >> 5], 1u << (myidx & 31));
+      wave_sync();
+      for (int w = lane; w < words; w += 64) p.bitmatrix[(int64_t)w * p.bm_stride_w + row] = words_s[wave][w];
+      wave_sync();
+    }
+  }
+  __syncthreads();
+  if (!q.col_sum) return;  // top-k only
+  // ---- phase 2: histogram out, offsets and ragged metadata ----
+  for (int e = threadIdx.x; e < E; e += kScanThreads) q.col_sum[e] = hist_s[e];
+  __threadfence_block();
+  __syncthreads();
+  ragged_metadata(q.col_sum, E, q.col_offs, q.r, q.want_ragged != 0);
+  __threadfence_block();
+  __syncthreads();
+  // ---- phase 3: stable ranks and the permutations ----
+  int total = q.col_offs[E];
+  for (int f = threadIdx.x; f < R; f += kScanThreads) {
+    const int e = eid_s[f];
+    int pos = -1;
+    if (e >= 0) {
+      int rank = 0;
+      for (int g = 0; g < f; ++g) rank += eid_s[g] == e ? 1 : 0;
+      pos = q.col_offs[e] + rank;
+      q.col_sorted[pos] = f;
+      if (q.gather_out) q.gather_out[pos] = f / k;
+      if (q.gammas_out) {
+        if (q.vals_bytes == 4)
+          static_cast<uint32_t*>(q.gammas_out)[pos] = val_s[f];
+        else
+          static_cast<uint16_t*>(q.gammas_out)[pos] = (uint16_t)val_s[f];
+      }
+    }
+    q.row_sorted[f] = pos;
+  }
+  // positions past the routed entries
+  for (int i = total + threadIdx.x; i < R; i += kScanThreads) {
+    q.col_sorted[i] = -1;
+    if (q.gather_out) q.gather_out[i] = -1;
+  }
+}
+
 struct ScatterParams {
   const int16_t* indx16;  // [T, k] (one of indx16 / indx32)
   const int32_t* indx32;
@@ -458,6 +604,30 @@ int32_t launch_topk(const TopkParams& p, int units, hipStream_t st) {
   return fail(TK_ERR_UNSUPPORTED, "tk_route: more than %d experts", kMaxExperts);
 }
 
+template <int DT>
+int32_t launch_small_dt(const SmallParams& q, hipStream_t st) {
+  const int epl = (q.t.E + 63) / 64;
+#define TK_EPL(N)                                                                                              \
+  if (epl <= N) {                                                                                              \
+    hipLaunchKernelGGL((route_small_kernel<DT, N>), dim3(1), dim3(kScanThreads), 0, st, q);                     \
+    return check_launch("route_small_kernel");                                                                 \
+  }
+  TK_EPL(1)
+  TK_EPL(2)
+  TK_EPL(4)
+  TK_EPL(8)
+  TK_EPL(16)
+  TK_EPL(32)
+#undef TK_EPL
+  return fail(TK_ERR_UNSUPPORTED, "tk_route: more than %d experts", kMaxExperts);
+}
+
+int32_t launch_small(const SmallParams& q, int dt, hipStream_t st) {
+  if (dt == TK_BF16) return launch_small_dt<TK_BF16>(q, st);
+  if (dt == TK_F16) return launch_small_dt<TK_F16>(q, st);
+  return launch_small_dt<TK_F32>(q, st);
+}
+
 }  // namespace
 }  // namespace tk
 
@@ -509,6 +679,30 @@ extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
   tp.fill_a = want_meta ? d->col_sorted_indx : nullptr;
   tp.fill_b = want_meta ? d->row_sorted_indx : nullptr;
   tp.fill_c = want_meta ? d->gather_indx : nullptr;
+  if ((int64_t)T * k <= kSmallEntries) {
+    // small batch: the whole pass in one launch
+    SmallParams sq;
+    sq.t = tp;
+    sq.t.partials = nullptr;
+    sq.t.fill_a = sq.t.fill_b = sq.t.fill_c = nullptr;
+    sq.col_sum = want_meta ? d->col_sum : nullptr;
+    sq.col_offs = col_offs;
+    sq.col_sorted = d->col_sorted_indx;
+    sq.row_sorted = d->row_sorted_indx;
+    sq.gather_out = d->gather_indx;
+    sq.gammas_out = d->vals ? d->gammas : nullptr;
+    sq.vals_bytes = (d->logits_dtype == TK_F32 || !d->logits) ? 4 : 2;
+    sq.want_ragged = d->slice_offs != nullptr;
+    sq.r.slice_offs = d->slice_offs;
+    sq.r.block_offs = d->block_offs;
+    sq.r.block_offs_stride = d->block_offs_stride;
+    sq.r.block_sched = d->block_schedule;
+    sq.r.block_sched_stride = d->block_schedule_stride;
+    sq.r.max_n_blocks = d->max_n_blocks;
+    if (want_meta && sq.want_ragged && (!d->block_offs || (!d->block_schedule && d->max_n_blocks > 0))) return fail(TK_ERR_INVALID, "tk_route: incomplete ragged outputs");
+    if (d->logits && d->logits_dtype != TK_F32 && d->logits_dtype != TK_BF16 && d->logits_dtype != TK_F16) return fail(TK_ERR_UNSUPPORTED, "tk_route: logits dtype %d", d->logits_dtype);
+    return launch_small(sq, d->logits ? d->logits_dtype : TK_F32, st);
+  }
   int32_t rc;
   if (d->logits_dtype == TK_F32 || !d->logits)
     rc = launch_topk<TK_F32>(tp, units, st);
