@@ -61,6 +61,31 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* x, int64_t 
   }
 }
 
+// Fast path of the k-way combine: bf16, no mask / scale, 8 columns (16 bytes) per thread, fp32 sum in j order.
+__global__ __launch_bounds__(256) void reduce_mid_bf16x8_kernel(const uint16_t* x, int64_t sx0, int64_t sx1, int64_t A, int K,
+                                                                int C8, uint16_t* y, int64_t sy0) {
+  const int64_t total = A * (int64_t)C8;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t a = i / C8;
+    const int c = (int)(i - a * C8) * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const uint16_t* src = x + a * sx0 + c;
+    for (int j = 0; j < K; ++j) {
+      const uint4 v = *reinterpret_cast<const uint4*>(src + j * sx1);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[2 * q] += bits_f32(w[q] << 16);
+        acc[2 * q + 1] += bits_f32(w[q] & 0xFFFF0000u);
+      }
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = (uint32_t)f32_to_bf16_bits(acc[2 * q]) | ((uint32_t)f32_to_bf16_bits(acc[2 * q + 1]) << 16);
+    *reinterpret_cast<uint4*>(y + a * sy0 + c) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 // Per-row dynamic quantisation to OCP e4m3: s = amax / 448 (1 for an all-zero row), q = sat(x / s).
 // One wave per row; the row is read twice (second pass hits L2).
 __global__ __launch_bounds__(256) void quant_fp8_rows_kernel(const uint16_t* x, int64_t stride_m, int64_t M, int64_t K,
@@ -116,8 +141,14 @@ extern "C" int32_t tk_reduce_mid(const void* x, int32_t dtype, int64_t A, int64_
   if (A == 0 || C == 0) return TK_OK;
   if (!x || !y) return fail(TK_ERR_INVALID, "tk_reduce_mid: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(A * C);
   const uint8_t* m = static_cast<const uint8_t*>(mask);
+  if (dtype == TK_BF16 && !mask && !scale && C % 8 == 0 && sx0 % 8 == 0 && sx1 % 8 == 0 && sy0 % 8 == 0 && K <= 0x7FFFFFFF && C <= 0x7FFFFFFF &&
+      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) {
+    hipLaunchKernelGGL(reduce_mid_bf16x8_kernel, dim3(grid_for(A * (C / 8))), dim3(256), 0, s, static_cast<const uint16_t*>(x), sx0, sx1, A,
+                       (int)K, (int)(C / 8), static_cast<uint16_t*>(y), sy0);
+    return check_launch("reduce_mid_bf16x8_kernel");
+  }
+  const int grid = grid_for(A * C);
   if (dtype == TK_BF16)
     hipLaunchKernelGGL(reduce_mid_kernel<TK_BF16>, dim3(grid), dim3(256), 0, s, x, sx0, sx1, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, y, sy0);
   else if (dtype == TK_F16)
