@@ -216,7 +216,13 @@ constexpr int kQuantities = 1 + kNumBlockSizes;  // rows, then row blocks of 16,
 // exchanged once through LDS.  offs0 (optional) and r.slice_offs (optional) receive the row offsets,
 // r.block_offs the block offsets.  Then every schedule slot finds its slice by binary search in the
 // block offsets, so a slice with thousands of blocks costs no more than an empty one.
+constexpr int kLdsOffsExperts = 1024;  // up to this many slices the offsets are also kept in LDS
+
 __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int E, int32_t* offs0, const RaggedOut r, bool want_ragged) {
+  // LDS copies: row 0 = slice offsets (read back by the single-launch router), rows 1.. = block offsets, which the
+  // schedule's binary search reads (seven dependent reads per slot; from global memory they dominated the kernel)
+  __shared__ int32_t offs_s[kQuantities][kLdsOffsExperts + 1];
+  const bool use_lds = E <= kLdsOffsExperts;
   __shared__ int wave_tot[kQuantities][kScanWaves + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nq = want_ragged ? kQuantities : 1;
@@ -259,6 +265,7 @@ __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int 
     for (int q = 0; q < kQuantities; ++q) {
       if (q < nq && i < E) {
         const int ex = carry[q] + wave_tot[q][wave] + inc[q] - v[q];
+        if (use_lds) offs_s[q][i] = ex;
         if (q == 0) {
           if (offs0) offs0[i] = ex;
           if (want_ragged) r.slice_offs[i] = ex;
@@ -271,6 +278,10 @@ __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int 
   }
   if (threadIdx.x == 0) {
     if (offs0) offs0[E] = carry[0];
+    if (use_lds) {
+#pragma unroll
+      for (int q = 0; q < kQuantities; ++q) offs_s[q][E] = carry[q];
+    }
     if (want_ragged) {
       r.slice_offs[E] = carry[0];
 #pragma unroll
@@ -282,7 +293,7 @@ __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int 
   __syncthreads();
 #pragma unroll
   for (int b = 0; b < kNumBlockSizes; ++b) {
-    const int32_t* offs = r.block_offs + b * r.block_offs_stride;
+    const int32_t* offs = use_lds ? offs_s[1 + b] : r.block_offs + b * r.block_offs_stride;
     int32_t* sched = r.block_sched + b * r.block_sched_stride;
     const int total = carry[1 + b];
     for (int i = threadIdx.x; i < r.max_n_blocks; i += kScanThreads) {
@@ -480,9 +491,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
   if (!q.col_sum) return;  // top-k only
   // ---- phase 2: histogram out, offsets and ragged metadata ----
   for (int e = threadIdx.x; e < E; e += kScanThreads) q.col_sum[e] = hist_s[e];
-  __threadfence_block();
-  __syncthreads();
-  ragged_metadata(q.col_sum, E, q.col_offs, q.r, q.want_ragged != 0);
+  ragged_metadata(hist_s, E, q.col_offs, q.r, q.want_ragged != 0);  // sizes straight from LDS
   __threadfence_block();
   __syncthreads();
   // ---- phase 3: stable ranks and the permutations ----
@@ -577,10 +586,10 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
 }
 
 // Rows one wave routes: one for small batches (latency), more as T grows so that the per-wave
-// histograms the scan has to walk stay at <= 256 rows of the workspace up to T = 4096 (<= 1024 beyond).
+// histograms the scan has to walk stay at <= 512 rows of the workspace up to T = 8192 (<= 1024 beyond).
 int rows_per_wave_for(int T) {
   int rpw = 1;
-  while ((int64_t)rpw * 256 < T && rpw < 16) rpw *= 2;
+  while ((int64_t)rpw * 512 < T && rpw < 16) rpw *= 2;
   while ((int64_t)rpw * 1024 < T) rpw *= 2;
   return rpw;
 }
