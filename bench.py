@@ -26,9 +26,9 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # HBM bytes one launch of the first expert GEMM moves at this workload, from two counter runs over this script
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from the 1 GiB copy of --calibrate-copy): 1819.1 MB read
-# + 103.1 MB written, against 1318.3 MB of algorithmic bytes.
-GEMM1_TRAFFIC_BYTES = 1.922e9
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from the 1 GiB copy of --calibrate-copy): 1346.6 MB read
+# + 94.4 MB written, against 1318.3 MB of algorithmic bytes.
+GEMM1_TRAFFIC_BYTES = 1.441e9
 
 
 def make_moe_weights(E, d_model, d_ff2, seed, device, n_copies=1):
@@ -312,7 +312,7 @@ def main():
                    "experts": E, "top_k": k, "w1": [E, d, f2], "w2": [E, f2 // 2, d]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM1_TRAFFIC_BYTES,
-                     "kernel": "moe_gemm_kernel (gather-GEMM W1 + bias + swiglu)", "kernel_ms": round(gemm1_ms, 4)},
+                     "kernel": "moe_gemm_mxn_kernel (gather-GEMM, tiled MXFP4 W1, bias, swiglu)", "kernel_ms": round(gemm1_ms, 4)},
     }
     # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
     layer_bytes = 2.19e9

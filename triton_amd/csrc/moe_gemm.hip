@@ -640,7 +640,7 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 // tile, so wider tiles cut the L2 -> L1 traffic, which is what bounds this kernel at prefill shapes.
 // WD / XD = depth of the weight register ring (2 or 4) / of the activation staging registers (1 or 2).
 // BLKM = rows of a row block in the ragged metadata (block_m).  A tile processes its block in passes of
-// BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 6 an expert of up to 192 rows is ONE tile (weights read
+// BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 5 an expert of up to 160 rows is ONE tile (weights read
 // once, no nearly empty second tile) and only larger blocks take a second pass.
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD, bool SWIGLU>
 __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams p) {
@@ -933,7 +933,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 // ------------------------------------------------------------------------------------------------
 // A few rows per expert: the kernel is bound by reading each active expert's weights once.  Every wave works
 // alone (no LDS, no barrier): it owns one 32-column weight fragment of one row block, streams the fragment's
-// K-stages through a six-deep register ring (12 KiB in flight per wave, up to sixteen waves per CU), reads its
+// K-stages through a four-deep register ring (8 KiB in flight per wave, up to sixteen waves per CU), reads its
 // rows' activations straight from L2 (each lane 64 contiguous bytes per stage), and issues 16x16x32 MFMAs
 // transposed like the prefill kernel (lane = column, 4 k-groups).  Within a stage lane group kg owns
 // k in [kg*32, kg*32 + 32): exactly one MX block and one 16-byte piece of the tiled layout.
@@ -1296,7 +1296,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->block_m == 16) return launch_mxd<1>(p, d->grid_m, swiglu, st);
     if (d->block_m == 32) return launch_mxd<2>(p, d->grid_m, swiglu, st);
     if (d->block_m == 64) return launch_mxn<64, 2, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
-    if (d->block_m == 256) return launch_mxn<256, 6, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
+    if (d->block_m == 256) return launch_mxn<256, 5, 2, 1, 2, 1>(p, d->grid_m, swiglu, st);
     return launch_mxn<128, 4, 2, 1, 4, 2>(p, d->grid_m, swiglu, st);
   }
   if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);

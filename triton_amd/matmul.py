@@ -283,7 +283,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     block_m = opt_flags.block_m
     if tiled:
         from .matmul_details.opt_flags import _get_opt_flags_constraints
-        if block_m == 128 and _get_opt_flags_constraints().get("block_m") is None and is_ragged and M <= 160 * n_slices:
+        if block_m == 128 and _get_opt_flags_constraints().get("block_m") is None and is_ragged and M <= 144 * n_slices:
             block_m = 256  # about 128 rows per expert: one tile per expert, the weights are read once
     elif block_m == 256:
         block_m = 128

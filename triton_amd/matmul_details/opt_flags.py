@@ -10,7 +10,7 @@ workgroup) and the weight format:
       32        128      256      4        128      128
       64        256      128      4        128      128
      128        256      128      4        128      128         prefill: ~128 rows per expert
-     256        256      128      4         -        -          pre-tiled MXFP4 only: a whole expert (<= 192 rows) per tile
+     256        256      128      4         -        -          pre-tiled MXFP4 only: a whole expert (<= 160 rows) per tile
 
 so only `block_m` can be forced; `block_n`, `block_k` and `num_warps` constraints must match the table.
 `split_k > 1` and `is_persistent=True` cannot be honoured and raise `InapplicableConstraint`, which is
@@ -27,7 +27,7 @@ TILE_TABLE = {  # narrow (4-bit / 8-bit) weights
     32: dict(block_n=128, block_k=256, num_warps=4),
     64: dict(block_n=256, block_k=128, num_warps=4),
     128: dict(block_n=256, block_k=128, num_warps=4),
-    256: dict(block_n=256, block_k=128, num_warps=4),  # pre-tiled MXFP4 weights only: one tile per expert of <= 192 rows
+    256: dict(block_n=256, block_k=128, num_warps=4),  # pre-tiled MXFP4 weights only: one tile per expert of <= 160 rows
 }
 TILE_TABLE_16BIT = {bm: dict(block_n=128, block_k=128, num_warps=4) for bm in TILE_TABLE}
 
