@@ -78,8 +78,19 @@ def _mx_weights(E, d, f2, g, scale=0.02):
     return w1q, w1s, w2q, w2s
 
 
+def _device_weights(layout, dev, w1q, w1s, w2q, w2s):
+    """Weights and scales on the device, either as the reference's strided tensors or converted once to the
+    layouts `matmul` prefers on this GPU (what a model loader does with make_default_matmul_mxfp4_w_layout)."""
+    W = {"w1": w1q.to(dev), "w1s": w1s.to(dev), "w2": w2q.to(dev), "w2s": w2s.to(dev)}
+    if layout == "tiled":
+        from bench import to_matmul_layout
+        W = to_matmul_layout(W)
+    return W
+
+
+@pytest.mark.parametrize("layout", ["strided", "tiled"])
 @pytest.mark.parametrize("T, skew", [(512, False), (1, True), (4, True), (16, True), (64, True)])
-def test_config3_4_mxfp4_reduced_experts(api, device, T, skew):
+def test_config3_4_mxfp4_reduced_experts(api, device, T, skew, layout):
     """gpt-oss shapes (d 2880, W1 [E, 2880, 5760], W2 [E, 2880, 2880], biases, top-4) with 16 experts so that
     the oracle finishes in seconds; decode batches use the skewed router of config 4."""
     g = torch.Generator().manual_seed(3 if skew else 2)
@@ -92,8 +103,9 @@ def test_config3_4_mxfp4_reduced_experts(api, device, T, skew):
     b1 = (torch.randn((E, f2), generator=g) * 0.01).to(torch.bfloat16)
     b2 = (torch.randn((E, d), generator=g) * 0.01).to(torch.bfloat16)
     dev = device
-    out, rdata, _ = _layer(api, dev, x, logits, k, w1q.to(dev), b1.to(dev), w2q.to(dev), b2.to(dev),
-                           api.PrecisionConfig(b_mx_scale=w1s.to(dev)), api.PrecisionConfig(b_mx_scale=w2s.to(dev)))
+    W = _device_weights(layout, dev, w1q, w1s, w2q, w2s)
+    out, rdata, _ = _layer(api, dev, x, logits, k, W["w1"], b1.to(dev), W["w2"], b2.to(dev),
+                           api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"]))
     ref, inter = omoe.moe_layer(x, logits, k, w1q, b1, w2q, b2, w1_mx_scale=w1s, w2_mx_scale=w2s, return_intermediates=True)
     assert_equal(inter["routing"].indx, rdata.expt_indx.to(torch.int32), "indx")
     assert_equal(inter["routing"].meta.col_sum, rdata.expt_hist, "histogram")
@@ -166,7 +178,8 @@ def test_legacy_matmul_ogs(api, device):
     assert_close(ref, out, what="matmul_ogs")
 
 
-def test_config3_full_shape_properties(api, device):
+@pytest.mark.parametrize("layout", ["strided", "tiled"])
+def test_config3_full_shape_properties(api, device, layout):
     """Full gpt-oss prefill shape (4096 tokens, 128 experts).  The oracle is too slow here, so the layer is
     checked through properties: (1) routing bit-exact against the oracle (cheap), (2) permuting the tokens
     permutes the output rows, (3) a token's output does not depend on which other tokens are in the batch
@@ -177,7 +190,11 @@ def test_config3_full_shape_properties(api, device):
     T, E, k, d, f2 = 4096, 128, 4, 2880, 5760
     x = torch.randn((T, d), generator=g).to(torch.bfloat16)
     logits = torch.randn((T, E), generator=g)
-    W = make_moe_weights(E, d, f2, seed=2, device=device)[0]
+    W0 = make_moe_weights(E, d, f2, seed=2, device=device)[0]
+    W = dict(W0)
+    if layout == "tiled":
+        from bench import to_matmul_layout
+        W = to_matmul_layout(W0)
     pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
     out, rdata, h = _layer(api, device, x, logits, k, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2)
     rr = ort.routing(logits, k)
@@ -194,6 +211,35 @@ def test_config3_full_shape_properties(api, device):
     for e in (0, 127):
         lo, hi = int(rr.ragged.slice_offs[e]), int(rr.ragged.slice_offs[e + 1])
         tok = rr.gather_indx[lo:hi].long()
-        he = omoe.matmul(x[tok], W["w1"][e:e + 1].cpu(), W["b1"][e:e + 1].cpu(), torch.tensor([hi - lo]), w_mx_scale=W["w1s"][e:e + 1].cpu())
+        he = omoe.matmul(x[tok], W0["w1"][e:e + 1].cpu(), W0["b1"][e:e + 1].cpu(), torch.tensor([hi - lo]), w_mx_scale=W0["w1s"][e:e + 1].cpu())
         ref = omoe.swiglu(he, 1.702, 7.0)
         assert_close(ref, h[lo:hi], maxtol=3e-2, what=f"expert {e} hidden")
+
+
+@pytest.mark.parametrize("T", [4, 256])
+def test_layer_graph_replays_match_eager(api, device, T):
+    """The layer captured in a HIP graph (what a serving loop replays): every replay, with new inputs copied
+    into the captured buffers and eager work and synchronisations in between, equals the eager result
+    bit for bit.  Covers the single-launch routing pass (T=4) and the three-kernel one (T=256)."""
+    from bench import capture
+    g = torch.Generator().manual_seed(11)
+    E, k, d, f2 = 16, 4, 2880, 5760
+    w1q, w1s, w2q, w2s = _mx_weights(E, d, f2, g)
+    W = _device_weights("tiled", device, w1q, w1s, w2q, w2s)
+    b1 = (torch.randn((E, f2), generator=g) * 0.01).to(torch.bfloat16).to(device)
+    b2 = (torch.randn((E, d), generator=g) * 0.01).to(torch.bfloat16).to(device)
+    pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
+    xs = torch.zeros((T, d), dtype=torch.bfloat16, device=device)
+    ls = torch.zeros((T, E), dtype=torch.float32, device=device)
+    run = lambda: _layer(api, device, xs, ls, k, W["w1"], b1, W["w2"], b2, pc1, pc2)[0]
+    xs.copy_(torch.randn((T, d), generator=g).to(torch.bfloat16))
+    ls.copy_(torch.randn((T, E), generator=g))
+    graph, out = capture(run)
+    for i in range(4):
+        xs.copy_(torch.randn((T, d), generator=g).to(torch.bfloat16))
+        ls.copy_(torch.randn((T, E), generator=g) + (i % 2) * torch.randn((E, ), generator=g))
+        eager = run().clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i} differs from the eager result"
