@@ -8,7 +8,7 @@ router -> gather-GEMM (+bias, swiglu) -> scatter-GEMM (+bias, gate weight) -> to
 seeded inputs resident in HBM.  Prints ONE JSON line; `value` is the layer's TFLOP/s (2*R*K*N over both
 GEMMs, R = routed rows).  `roofline` covers the dominant kernel (the first expert GEMM), timed live with
 HIP events on the launch stream; `cpu_baseline` is the CPU oracle on a bounded sample of the same
-workload; `extra` carries the decode (config 4) and MX round-trip (config 2) figures.
+workload; `extra` carries the FP8 (config 5), decode (config 4) and MX round-trip (config 2) figures.
 """
 from __future__ import annotations
 
@@ -228,6 +228,49 @@ def bench_mx(device, steps, warmup):
                 frac_hbm_dequant=round(nbytes / ms_d / 1e6 / PEAK_HBM_GBPS, 4))
 
 
+def bench_fp8(device, steps, warmup):
+    """Config 5 (Mixtral-style FP8) at full size: 8192 tokens, top-2 of 8 experts, W1 [8, 4096, 28672] and
+    W2 [8, 14336, 4096] in e4m3 with per-output-channel fp32 scales, activations quantised per token to e4m3
+    before each GEMM.  One step = router, quantise, GEMM1 + swiglu, quantise, GEMM2 * gate, combine."""
+    from triton_kernels.legacy import routing
+    from triton_kernels.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
+    from triton_kernels.numerics_details.rowwise_fp8 import quantize_fp8_rowwise
+    from triton_kernels.reduce import reduce
+    from triton_kernels.swiglu import swiglu_fn
+    T, d, E, k, f2 = 8192, 4096, 8, 2, 28672
+    torch.manual_seed(4)
+    x = torch.randn((T, d), device=device).to(torch.bfloat16)
+    logits = torch.randn((T, E), device=device)
+
+    def qw(kdim, ndim):  # K-major e4m3 weights [E, K, N] (stride 1 along K) and their column scales [E, N]
+        q = torch.empty((E, ndim, kdim), dtype=torch.float8_e4m3fn, device=device)
+        s = torch.empty((E, ndim), dtype=torch.float32, device=device)
+        for e in range(E):
+            w = torch.randn((ndim, kdim), device=device) * 0.02
+            s[e] = w.abs().amax(dim=1) / 448.0
+            q[e] = (w / s[e][:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
+        return q.transpose(1, 2), s
+
+    w1, s1 = qw(d, f2)
+    w2, s2 = qw(f2 // 2, d)
+    act = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0))
+
+    def step():
+        rdata, _, scatter = routing(logits, k)
+        xq, sx = quantize_fp8_rowwise(x)
+        h = matmul(xq, w1, None, rdata.expt_data, gather_indx=rdata.token_indx, fused_activation=act,
+                   precision_config=PrecisionConfig(a_mx_tensor_scale=sx, b_mx_tensor_scale=s1, out_dtype=torch.bfloat16))
+        hq, sh = quantize_fp8_rowwise(h)
+        y = matmul(hq, w2, None, rdata.expt_data, scatter_indx=scatter.dst_indx, gammas=rdata.gate_scal,
+                   precision_config=PrecisionConfig(a_mx_tensor_scale=sh, b_mx_tensor_scale=s2, out_dtype=torch.bfloat16))
+        return reduce(y.view(T, k, -1), dim=1)[0]
+
+    ms = time_steps(step, steps, warmup)
+    flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
+    return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8",
+                frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -320,7 +363,8 @@ def main():
     rec["layer_roofline"] = {"t_roof_ms": round(t_roof_ms, 4), "frac": round(t_roof_ms / ms, 4),
                              "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1)}
     if not args.no_extra:
-        rec["extra"] = {"decode_config4": bench_decode(device, max(5, args.steps), args.warmup),
+        rec["extra"] = {"fp8_config5": bench_fp8(device, max(5, args.steps // 2), 2),
+                        "decode_config4": bench_decode(device, max(5, args.steps), args.warmup),
                         "mx_round_trip_config2": bench_mx(device, max(5, args.steps), args.warmup)}
     if not args.no_cpu:
         rec["cpu_baseline"] = cpu_baseline()

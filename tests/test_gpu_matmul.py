@@ -129,6 +129,75 @@ def test_fused_swiglu(mods, device, m, n, k, wkind, block_m, opts):
     assert_close(omoe.swiglu(y2.cpu(), opts[0], opts[1]), s2, maxtol=1e-2, what="standalone swiglu")
 
 
+@pytest.mark.parametrize("kind", ["mxfp8_e4m3", "mxfp8_e5m2", "mxfp4"])
+@pytest.mark.parametrize("wkind, swiglu, scatter", [("bf16", False, False), ("mxfp4_tiled", True, False), ("mxfp4", False, True)])
+def test_mx_output_epilogue(mods, device, kind, wkind, swiglu, scatter):
+    """`Epilogue(FnSpecs(QUANTIZE_MXFP8 | QUANTIZE_MXFP4))` + `c_mx_scale` (reference test: tests/test_matmul.py:560-573,
+    checked at :627-643 by dequantising and comparing with maxtol 4e-1 / rmstol 4e-2 against the quantised reference).
+    Two checks: (1) the values and scales are bit for bit the oracle's quantisation of the GEMM's own bf16 output;
+    (2) dequantised, they meet the reference's tolerance against the oracle's GEMM -> quantise -> dequantise."""
+    mm, sw, tensor = mods
+    from triton_amd.numerics_details.mxfp import quantize_mxfp4_fn, quantize_mxfp8_fn
+    g = torch.Generator().manual_seed(17)
+    m, n, k, n_slices = 300, 512, 416, 6
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, wkind, g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    sc = torch.randperm(m, generator=g).to(torch.int32) if scatter else None
+    n_out = n // 2 if swiglu else n
+    out_dtype = {"mxfp8_e4m3": torch.float8_e4m3fn, "mxfp8_e5m2": torch.float8_e5m2, "mxfp4": torch.uint8}[kind]
+    name, fn = (mm.FnName.QUANTIZE_MXFP4.name, quantize_mxfp4_fn) if kind == "mxfp4" else (mm.FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn)
+    epi = mm.Epilogue(mm.FnSpecs(name, fn, (), ()), tuple(), tuple(), effective_itemsize=6.0)
+    c_scale = torch.full((m, n_out // 32), 0xFF, dtype=torch.uint8, device=device)
+    kw = dict(fused_activation=act, scatter_indx=None if sc is None else sc.to(device))
+    pc = mm.PrecisionConfig(b_mx_scale=W["scale_dev"], c_mx_scale=c_scale, out_dtype=out_dtype)
+    yq = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=pc, epilogue=epi, **kw)
+    assert yq.dtype == out_dtype and yq.shape == (m, n_out // 2 if kind == "mxfp4" else n_out)
+    assert pc.c_mx_scale is c_scale and pc.c_value_pack_factor == (2 if kind == "mxfp4" else 1)
+    y = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]), **kw)
+    q_ref, s_ref = omx.downcast_to_mxfp(y.cpu(), out_dtype, axis=-1)
+    assert torch.equal(q_ref.view(torch.uint8), yq.cpu().view(torch.uint8)), "values are not the quantisation of the bf16 result"
+    assert torch.equal(s_ref, c_scale.cpu()), "scales are not the quantisation of the bf16 result"
+    h = omoe.matmul(x, W["w_cpu"], bias, sizes, w_mx_scale=W["scale_cpu"], scatter_indx=sc)
+    if swiglu:
+        h = omoe.swiglu(h, 1.702, 7.0)
+    ref = omx.upcast_from_mxfp(*omx.downcast_to_mxfp(h, out_dtype, axis=-1), torch.bfloat16, axis=-1)
+    got = omx.upcast_from_mxfp(yq.cpu(), c_scale.cpu(), torch.bfloat16, axis=-1)
+    if kind == "mxfp4":
+        # 3-bit magnitudes: an fp32-vs-bf16 rounding difference next to a decision threshold moves a value by a whole
+        # e2m1 step (up to 100 % of a small value), so the max-error bound of the fp8 case does not apply; the
+        # reference has no MXFP4-output test.  Bounded by how many elements differ and by the rms error.
+        from oracle.checks import rel_errors
+        differing = (ref.float() != got.float()).float().mean().item()
+        _, rms = rel_errors(ref, got)
+        assert differing <= 0.03 and rms <= 1e-1, f"mxfp4 output: {differing:.4f} of the elements differ, rms {rms:.4g}"
+    else:
+        assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
+
+
+@pytest.mark.parametrize("wkind", ["mxfp4", "mxfp4_tiled"])
+def test_cdna4_scale_layout_accepted(mods, device, wkind):
+    """Scales pre-shuffled with the reference's `CDNA4MXScaleLayout` (what its default helper returns on this GPU,
+    tensor_details/layout.py:43-54) give the same result, bit for bit, as the same scales in the kernel's own order."""
+    mm, _, tensor = mods
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
+    g = torch.Generator().manual_seed(23)
+    m, n, k, n_slices = 300, 416, 576, 5
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16).to(device)
+    W = _make_w(n_slices, k, n, wkind, g, device)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    cd = convert_layout(wrap_torch_tensor(W["scale_cpu"].to(device)), CDNA4MXScaleLayout())
+    y_ref = mm.matmul(x, W["w_dev"], None, md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]))
+    for _ in range(2):  # the second call takes the cached conversion
+        y = mm.matmul(x, W["w_dev"], None, md, precision_config=mm.PrecisionConfig(b_mx_scale=cd))
+        assert torch.equal(y, y_ref)
+
+
 def test_zero_sized(mods, device):
     mm, _, tensor = mods
     for m, n, k in [(0, 5, 7), (5, 0, 7)]:
@@ -145,6 +214,11 @@ def test_rejected_options(mods, device):
         mm.matmul(x, w, None, betas=torch.ones(4, device=device))
     with pytest.raises(NotImplementedError):
         mm.matmul(x, w, None, c_acc_in=torch.zeros((4, 16), device=device))
+    with pytest.raises(NotImplementedError):  # NVFP4 output (float8 block scales) is a Blackwell format
+        mm.matmul(x, w, None, epilogue=mm.Epilogue(mm.FnSpecs(mm.FnName.QUANTIZE_NVFP4.name, object(), (), ()), (), (), 2.0))
+    with pytest.raises(ValueError):  # an MX epilogue without a scale tensor to fill
+        mm.matmul(x, w, None, precision_config=mm.PrecisionConfig(out_dtype=torch.float8_e4m3fn),
+                  epilogue=mm.Epilogue(mm.FnSpecs(mm.FnName.QUANTIZE_MXFP8.name, object(), (), ()), (), (), 6.0))
     with pytest.raises(mm.InapplicableConstraint):
         with mm.scoped_opt_flags_constraints({"split_k": 2}):
             mm.matmul(x, w, None)

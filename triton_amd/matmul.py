@@ -12,8 +12,9 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
     fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
 
 Options of the reference signature that this build rejects with NotImplementedError: ragged-K
-(`b_ragged_metadata`), `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, MX-output epilogues, flexpoint
-scales, batched 3-D activations, split-k.
+(`b_ragged_metadata`), `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
+scales, batched 3-D activations, split-k.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
+MX quantiser kernel on the same stream.
 """
 from __future__ import annotations
 
@@ -28,7 +29,8 @@ from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_op
                                         scoped_opt_flags_constraints, set_idle_sms)
 from .numerics import InFlexData, OutFlexData
 from .specialize import FnSpecs
-from .tensor import FP4, RaggedTensorMetadata, Tensor, torch_dtype_to_dtype, wrap_torch_tensor
+from .tensor import FP4, RaggedTensorMetadata, Tensor, convert_layout, torch_dtype_to_dtype, wrap_torch_tensor
+from .tensor_details.layout_details.cdna4_scale import CDNA4MXScaleLayout
 from .tensor_details.layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
 from .tensor_details.layout_details.strided import StridedLayout
 
@@ -112,6 +114,53 @@ def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
     return w.transpose(-1, -2).contiguous().transpose(-1, -2)
 
 
+def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
+                   fused_activation, epilogue):
+    """`Epilogue(FnSpecs(QUANTIZE_MXFP8 | QUANTIZE_MXFP4, ...))` with `precision_config.c_mx_scale`
+    (triton_kernels/matmul.py:53-56,364-369,500-505; kernel side matmul_details/_matmul.py:593-637): the output is
+    quantised along N in blocks of 32, values in `out_dtype` (float8 or packed e2m1 in uint8) and one e8m0 scale
+    byte per block written to `c_mx_scale` [rows, ceil(N_out / 32)].  Here the GEMM writes bf16 and the MX
+    quantiser kernel follows on the same stream, so the values are quantised from the bf16-rounded result (the
+    reference quantises the fp32 accumulator: a code can differ by one step where the bf16 rounding crosses a
+    quantisation threshold)."""
+    import dataclasses
+    from .numerics_details.mxfp import downcast_to_mxfp
+    scale_out = precision_config.c_mx_scale
+    if scale_out is None:
+        raise ValueError("an MX-quantising epilogue needs precision_config.c_mx_scale to receive the block scales")
+    if precision_config.c_microblock_size not in (None, MXFP_BLOCK_SIZE):
+        raise NotImplementedError(f"output microblock size {precision_config.c_microblock_size} is not supported (32 only)")
+    fp4 = epilogue.specs.name == FnName.QUANTIZE_MXFP4.name
+    out_dtype = precision_config.out_dtype
+    if out_dtype not in ((torch.uint8, ) if fp4 else (torch.float8_e4m3fn, torch.float8_e5m2)):
+        raise ValueError(f"epilogue {epilogue.specs.name} does not produce out_dtype {out_dtype}")
+    if isinstance(scale_out, Tensor):
+        if not isinstance(scale_out.storage.layout, StridedLayout):
+            raise NotImplementedError(f"output scale layout {type(scale_out.storage.layout).__name__} is not supported")
+        scale_data = scale_out.storage.data
+    else:
+        scale_data = scale_out
+    assert scale_data.dtype == torch.uint8, f"Unsupported output microscale dtype {scale_data.dtype}"
+    plain = dataclasses.replace(precision_config, c_mx_scale=None, out_dtype=torch.bfloat16)
+    y = matmul(a, b, bias, a_ragged_metadata, None, gather_indx, scatter_indx, plain, None, gammas, None, None, None,
+               fused_activation, None, None)
+    n_out = y.shape[-1]
+    if n_out % MXFP_BLOCK_SIZE != 0:
+        raise NotImplementedError(f"MX-quantised output needs N_out % 32 == 0 (got {n_out})")
+    assert tuple(scale_data.shape[-2:]) == (y.shape[0], n_out // MXFP_BLOCK_SIZE), \
+        f"c_mx_scale must be [{y.shape[0]}, {n_out // MXFP_BLOCK_SIZE}], got {tuple(scale_data.shape)}"
+    vals, scales = downcast_to_mxfp(y, out_dtype, axis=-1)
+    scale_data.view(scales.shape).copy_(scales)
+    precision_config.c_mx_scale = scale_out
+    precision_config.c_microblock_size = MXFP_BLOCK_SIZE
+    precision_config.c_value_pack_factor = 2 if fp4 else 1
+    if c is not None:
+        assert tuple(c.shape[-2:]) == tuple(vals.shape) and c.dtype == vals.dtype
+        c.view(vals.shape).copy_(vals)
+        return c
+    return vals
+
+
 def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
            b_ragged_metadata: RaggedTensorMetadata | None = None, gather_indx: torch.Tensor | None = None,
            scatter_indx: torch.Tensor | None = None, precision_config: PrecisionConfig | None = None,
@@ -140,8 +189,11 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         fused_activation = FusedActivation(FnSpecs.default(), tuple())
     if epilogue is None:
         epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+    if epilogue.specs.name in (FnName.QUANTIZE_MXFP8.name, FnName.QUANTIZE_MXFP4.name):
+        return _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
+                              fused_activation, epilogue)
     if epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
-        raise NotImplementedError("MX-output / custom epilogues are not supported")
+        raise NotImplementedError(f"epilogue {epilogue.specs.name!r} is not supported (MXFP8 / MXFP4 output quantisation only)")
     if not _flex_is_trivial(precision_config.flex_ctx):
         raise NotImplementedError("flexpoint scales are not supported; use a/b_mx_tensor_scale for fp8 scales")
     if precision_config.a_mx_scale is not None:
@@ -160,6 +212,15 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         raise NotImplementedError(f"weight layout {type(b.storage.layout).__name__} is not supported")
     if b_scale is not None and not isinstance(b_scale, Tensor):
         b_scale = wrap_torch_tensor(b_scale)
+    if b_scale is not None and isinstance(b_scale.storage.layout, CDNA4MXScaleLayout):
+        # the reference's scale pre-shuffle: converted once to the order that goes with the values' layout and
+        # kept on the wrapper (weights are static; re-wrap the tensor after changing its storage in place)
+        want = GFX950MXScaleLayout() if tiled else StridedLayout(-2)
+        cached = getattr(b_scale, "_tk_converted", None)
+        if cached is None or cached[0] != want:
+            cached = (want, convert_layout(b_scale, want))
+            b_scale._tk_converted = cached
+        b_scale = cached[1]
     if b_scale is not None:
         if tiled != isinstance(b_scale.storage.layout, GFX950MXScaleLayout):
             raise NotImplementedError("tiled MXFP4 values go with tiled scales (convert both with convert_layout)")

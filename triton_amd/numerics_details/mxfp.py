@@ -27,6 +27,23 @@ MXFP_BLOCK_SIZE = _BlockSize(32)
 NVFP_BLOCK_SIZE = _BlockSize(16)
 
 
+class _EpilogueFn:
+    """Token carried by `Epilogue(FnSpecs(FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn, (), ()), ...)`; the
+    reference passes a device function here (`triton_kernels/numerics_details/mxfp.py:432-434`), `matmul` in this
+    build recognises the epilogue by its name and runs the MX quantiser kernel."""
+
+    def __init__(self, name):
+        self.name = name
+
+    def __repr__(self):
+        return self.name
+
+
+quantize_mxfp8_fn = _EpilogueFn("_quantize_mxfp8_fn")
+quantize_mxfp4_fn = _EpilogueFn("_quantize_mxfp4_fn")
+quantize_nvfp4_fn = _EpilogueFn("_quantize_nvfp4_fn")
+
+
 class DequantScaleRoundingMode(Enum):
     ROUND_UP = 0  # 2^ceil(log2(max / max_q)): never clips the block maximum
     ROUND_DOWN = 1  # 2^floor(log2(max / max_pow2_q)): the OCP rule

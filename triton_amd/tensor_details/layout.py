@@ -3,13 +3,16 @@
 Two families exist on gfx950 in this build: the strided layout (what `downcast_to_mxfp` returns) and the
 pre-tiled MXFP4 pair `GFX950MXValueLayout` / `GFX950MXScaleLayout`, which the default-layout helpers return
 for weights whose MX axis is K, as the reference's helpers return its architecture-specific layouts
-(layout.py:26-54).  Both are accepted by `matmul`; the tiled pair is the fast path.
+(layout.py:26-54).  Both are accepted by `matmul`; the tiled pair is the fast path.  `CDNA4MXScaleLayout`, the
+reference's own scale pre-shuffle for this GPU, is accepted too: `matmul` converts such scales once to the order
+that goes with the weight values' layout.
 """
 from .layout_details.base import Layout
+from .layout_details.cdna4_scale import CDNA4MXScaleLayout
 from .layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
 from .layout_details.strided import StridedLayout
 
-__all__ = ["Layout", "StridedLayout", "GFX950MXValueLayout", "GFX950MXScaleLayout"]
+__all__ = ["Layout", "StridedLayout", "GFX950MXValueLayout", "GFX950MXScaleLayout", "CDNA4MXScaleLayout"]
 
 
 def make_default_matmul_mxfp4_w_layout(mx_axis: int, **_unused):
