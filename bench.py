@@ -251,8 +251,13 @@ def bench_fp8(device, steps, warmup):
             q[e] = (w / s[e][:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
         return q.transpose(1, 2), s
 
+    from triton_kernels.tensor import convert_layout, wrap_torch_tensor
+    from triton_kernels.tensor_details.layout import make_default_matmul_fp8_w_layout
     w1, s1 = qw(d, f2)
     w2, s2 = qw(f2 // 2, d)
+    # converted once, as a model loader would, to the layout `matmul` prefers for e4m3 weights on this GPU
+    w1 = convert_layout(wrap_torch_tensor(w1), make_default_matmul_fp8_w_layout())
+    w2 = convert_layout(wrap_torch_tensor(w2), make_default_matmul_fp8_w_layout())
     act = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0))
 
     def step():

@@ -178,6 +178,63 @@ def test_mx_output_epilogue(mods, device, kind, wkind, swiglu, scatter):
         assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
 
 
+def _fp8_operands(m, n, k, n_slices, g):
+    """e4m3 activations with one fp32 scale per row, e4m3 weights with one fp32 scale per (expert, column)."""
+    x = torch.randn((m, k), generator=g)
+    sx = x.abs().amax(dim=1).clamp_min(1e-6) / 448.0
+    xq = (x / sx[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
+    w = torch.randn((n_slices, k, n), generator=g) * 0.05
+    sw = w.abs().amax(dim=1) / 448.0  # [E, N]
+    wq = (w / sw[:, None, :]).clamp(-448, 448).to(torch.float8_e4m3fn)
+    return xq, sx, wq, sw
+
+
+@pytest.mark.parametrize("m, n, k", [(300, 400, 416), (1000, 704, 832), (2100, 512, 1024), (64, 96, 16)])
+@pytest.mark.parametrize("layout, block_m", [("strided", 16), ("strided", 128), ("tiled", 128), ("tiled", 256)])
+@pytest.mark.parametrize("do_gather, do_scatter, do_gamma, swiglu", [(False, False, False, False), (True, False, True, True),
+                                                                      (False, True, True, False), (True, True, False, True)])
+def test_matmul_fp8(mods, device, m, n, k, layout, block_m, do_gather, do_scatter, do_gamma, swiglu):
+    """e4m3 x e4m3 with per-row and per-column fp32 scales (config 5's operands; the reference's hooks:
+    matmul.py:620-626, _matmul.py:363-382,507-517).  PARITY UNPINNED by the reference's tests; the oracle
+    dequantises both operands and runs the pinned GEMM oracle.  Strided K-contiguous weights and the tiled FP8 layout."""
+    mm, sw_mod, tensor = mods
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import make_default_matmul_fp8_w_layout
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    n_slices = 6
+    xq, sx, wq, sw = _fp8_operands(m, n, k, n_slices, g)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    gi = torch.randint(0, m, (m, ), generator=g).to(torch.int32) if do_gather else None
+    sc = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    gam = (torch.rand((m, ), generator=g) + 0.5) if do_gamma else None
+    wd = wq.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)  # stride 1 along K
+    if layout == "tiled":
+        wd = convert_layout(wrap_torch_tensor(wd), make_default_matmul_fp8_w_layout())
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw_mod.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    pc = mm.PrecisionConfig(a_mx_tensor_scale=sx.to(device), b_mx_tensor_scale=sw.to(device), out_dtype=torch.bfloat16)
+    dv = lambda t: None if t is None else t.to(device)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(xq.to(device), wd, bias.to(device), md, gather_indx=dv(gi), scatter_indx=dv(sc), gammas=dv(gam),
+                      precision_config=pc, fused_activation=act)
+    # the oracle applies the gate weight inside matmul; with swiglu the kernel applies it after the activation
+    ref = omoe.matmul(xq, wq, bias, sizes, gather_indx=gi, scatter_indx=None if swiglu else sc, gammas=None if swiglu else gam,
+                      x_row_scale=sx, w_col_scale=sw, out_dtype=torch.float32 if swiglu else torch.bfloat16)
+    if swiglu:
+        ref = omoe.swiglu(ref, 1.702, 7.0).float()
+        if gam is not None:
+            ref = ref * gam[:, None]
+        ref = ref.to(torch.bfloat16)
+        if sc is not None:
+            out = torch.zeros_like(ref)
+            out[sc.long()] = ref
+            ref = out
+    assert y.shape == ref.shape
+    assert_close(ref, y, maxtol=3e-2 if swiglu else 2e-2, what="fp8 y")
+    assert_allclose_gate(ref, y, what="fp8 y", max_bad_frac=1e-4 if swiglu else 0.0)
+
+
 @pytest.mark.parametrize("wkind", ["mxfp4", "mxfp4_tiled"])
 def test_cdna4_scale_layout_accepted(mods, device, wkind):
     """Scales pre-shuffled with the reference's `CDNA4MXScaleLayout` (what its default helper returns on this GPU,

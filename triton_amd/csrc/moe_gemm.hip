@@ -1104,6 +1104,238 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc, expert, off_m, start_m, eM, F * 32, F * 32 + 32 <= N, 0, lr, kg);
 }
 
+// ------------------------------------------------------------------------------------------------
+// e4m3 weights in a tile-native layout x e4m3 activations (prefill): FP8 MFMA, no conversion in the loop
+// ------------------------------------------------------------------------------------------------
+// Weight layout (built once per model by the host from the K-contiguous form): per expert, per fragment F of 32
+// output columns (N padded to 32), per K-stage s of 128 (K padded to 128 with zero weights): one 4 KiB block
+// [q:4][lane:64][16 B]; lane = h*32 + lr holds the e4m3 bytes of column F*32 + lr for
+// k in [s*128 + (q/2)*64 + h*32 + (q%2)*16, +16): pieces 2t and 2t+1 of a lane are the 32 consecutive bytes it
+// feeds to the v_mfma_f32_32x32x64_f8f6f4 of K-step t.  The activation rows (gathered, one byte per element)
+// are staged through LDS with a 144-byte row pitch and read back as the same 32 consecutive bytes per lane, so
+// both operands put the same k in the same byte position whatever order the instruction sums them in.
+// Per-row and per-column fp32 scales, bias, activation and gate weight are applied by the shared epilogue.
+//
+// Structure as in the MXFP4 prefill kernel: four waves, each owning NFW column fragments whose weights go
+// global memory -> register ring (WD stages deep) -> MFMA, all sharing the MFW row fragments of the tile through
+// an LDS double buffer; two K-steps per stage; one workgroup barrier per stage, in step 1; persistent grid with
+// XCD-aware rounds and (expert, column tile, row block) tile order.
+typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
+
+template <int BLKM, int MFW, int NFW, int WD, int XD, bool SWIGLU>
+__global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
+  typedef Frag<32> FR;
+  constexpr int FM = 32, BM = MFW * 32, BN = 128 * NFW, KC = 128;
+  static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2), "ring depths");
+  constexpr int XPITCH = KC + 16;
+  constexpr int XBYTES = BM * XPITCH;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int nw = __builtin_amdgcn_readfirstlane(tid >> 6);  // column quarter of the tile
+  const int lr = lane & 31, h = lane >> 5;
+  const int K = p.K, N = p.N;
+  const int nst = p.w_nst;
+  const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
+  for (int round0 = 0; round0 < live; round0 += (int)gridDim.x) {
+  const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
+  if ((int)blockIdx.x >= in_round) break;
+  const int pid = round0 + xcd_remap(blockIdx.x, in_round);
+  int expert, blk_off, start_m, eM, pid_n;
+  if (p.slice_sizes) {
+    expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
+    const int first = p.block_offs[expert];
+    const int nb = p.block_offs[expert + 1] - first;
+    const int local = pid - first * p.grid_n;
+    pid_n = local / nb;
+    blk_off = (local - pid_n * nb) * BLKM;
+    start_m = p.slice_offs[expert];
+    eM = p.slice_sizes[expert];
+  } else {
+    pid_n = pid % p.grid_n;
+    expert = 0;
+    blk_off = (pid / p.grid_n) * BLKM;
+    start_m = 0;
+    eM = p.M;
+  }
+  const int blk_rows = (eM - blk_off) < BLKM ? (eM - blk_off) : BLKM;
+  for (int pass_off = 0; pass_off < blk_rows; pass_off += BM) {
+  const int off_m = blk_off + pass_off;
+  const int rows = (blk_rows - pass_off) < BM ? (blk_rows - pass_off) : BM;
+  const int nj = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW)
+
+  // ---- activation staging: piece j of this thread = row 32 j + tid/8, 16-byte chunk tid%8 of the stage ----
+  const int xc = tid & 7;
+  const uint8_t* xptr[MFW];
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    int row = off_m + (tid >> 3) + 32 * j;
+    row = row < eM ? row : eM - 1;
+    const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
+    xptr[j] = p.x + src * p.x_stride_m;
+  }
+  const int xlds0 = (tid >> 3) * XPITCH + xc * 16;  // piece j at xlds0 + j*32*XPITCH
+
+  const int nfr = (N + 31) >> 5;
+  const uint8_t* wptr[NFW];
+#pragma unroll
+  for (int f = 0; f < NFW; ++f) {
+    int F = pid_n * (BN / 32) + nw * NFW + f;
+    F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
+    wptr[f] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 4096 + lane * 16;
+  }
+
+  typename FR::acc_t acc[NFW][MFW];
+#pragma unroll
+  for (int f = 0; f < NFW; ++f)
+#pragma unroll
+    for (int j = 0; j < MFW; ++j)
+#pragma unroll
+      for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
+
+  u32x4_t xreg[XD][MFW];
+  i32x8_t wreg[WD][NFW][2];  // [ring slot][column fragment][K-step]
+  i32x8_t xf[2][MFW];        // [K-step][row fragment]
+
+  // Loads are unconditional: rows past the last valid row re-read it, k past K re-reads the row's last 16 bytes
+  // (the padded weights there are zero), stages past the last one re-read the last stage.
+  auto load_x_piece = [&](int j, int s, int slot) __attribute__((always_inline)) {
+    int k0 = s * KC + xc * 16;
+    k0 = k0 < K - 16 ? k0 : K - 16;
+    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0);
+  };
+  auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 32 * XPITCH) = xreg[slot][j];
+  };
+  auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
+    constexpr int SL = decltype(slot_c)::value;
+    s = s < nst ? s : nst - 1;
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 4096 + (2 * t) * 1024);
+        const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 4096 + (2 * t + 1) * 1024);
+        wreg[SL][f][t] = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+  };
+  auto read_xf = [&](int buf, int t, int j, i32x8_t (&out)[MFW]) __attribute__((always_inline)) {
+    const uint8_t* a = lds + buf * XBYTES + (j * FM + lr) * XPITCH + t * 64 + h * 32;
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(a);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(a + 16);
+    out[j] = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  template_int<0> S0;
+  template_int<1> S1;
+  template_int<2> S2;
+  template_int<3> S3;
+
+  // One K-stage (two K-steps of 64).  NJ = row fragments with valid rows; WS = c % WD = weight ring slot, the LDS
+  // buffer is WS & 1.  Step 0 interleaves, between its MFMAs: the LDS reads of step 1's activations, the LDS
+  // writes of the next stage's activations (other buffer) with the refill of their staging registers, and the
+  // weight loads WD-1 stages ahead.  Step 1: after its first MFMA every wave has read all it needs from this
+  // stage's buffer and written its share of the next one; barrier; then the reads of the next stage's step 0.
+  auto stage = [&](auto nj_c, auto ws_c, int c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    constexpr int WS = decltype(ws_c)::value;
+    constexpr int PAR = WS & 1;
+    using WSL = template_int<(WS + WD - 1) % WD>;
+    constexpr int XS = (WS + 1) % XD;
+    constexpr int NM = NJ * NFW;
+    constexpr int NOPS = 2 * NJ + 1;
+    static_for<0, 2>([&](auto t_c) __attribute__((always_inline)) {
+      constexpr int t = decltype(t_c)::value;
+      auto op = [&](auto o_c) __attribute__((always_inline)) {
+        constexpr int o = decltype(o_c)::value;
+        if constexpr (t == 0) {
+          if constexpr (o < NJ) {
+            read_xf(PAR, 1, o, xf[1]);
+          } else if constexpr (o < 2 * NJ) {
+            store_x_piece(o - NJ, PAR ^ 1, XS);
+            load_x_piece(o - NJ, c + 1 + XD, XS);
+          } else {
+            load_w(WSL{}, c + WD - 1);
+          }
+        } else {
+          if constexpr (o < NJ) read_xf(PAR ^ 1, 0, o, xf[0]);
+        }
+      };
+      static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_c)::value;
+        constexpr int j = m / NFW, f = m % NFW;
+        acc[f][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wreg[WS][f][t], xf[t][j], acc[f][j], 0, 0, 0, 0, 0, 0);
+        if constexpr (t == 1 && m == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        }
+        static_for<(m * NOPS) / NM, ((m + 1) * NOPS) / NM>(op);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+
+  auto run = [&](auto nj_c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    // Prologue: stage 0 without overlap; the loads left in flight are issued in the order the steady state leaves
+    // them in at the top of a stage (activations, then weights, of stage 1, then of stage 2).
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(S0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1 % XD); });
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (WD == 4) {
+      load_w(S1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (XD == 2) {
+      static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 2, 0); });
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (WD == 4) {
+      load_w(S2, 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { read_xf(0, 0, decltype(jc)::value, xf[0]); });
+    __builtin_amdgcn_sched_barrier(0);
+    int c = 0;
+    if constexpr (WD == 4) {
+      for (; c + 3 < nst; c += 4) {
+        stage(nj_c, S0, c);
+        stage(nj_c, S1, c + 1);
+        stage(nj_c, S2, c + 2);
+        stage(nj_c, S3, c + 3);
+      }
+      if (c < nst) stage(nj_c, S0, c);
+      if (c + 1 < nst) stage(nj_c, S1, c + 1);
+      if (c + 2 < nst) stage(nj_c, S2, c + 2);
+    } else {
+      for (; c + 1 < nst; c += 2) {
+        stage(nj_c, S0, c);
+        stage(nj_c, S1, c + 1);
+      }
+      if (c < nst) stage(nj_c, S0, c);
+    }
+  };
+  static_for<1, MFW + 1>([&](auto n_c) __attribute__((always_inline)) {
+    if (nj == decltype(n_c)::value) run(n_c);
+  });
+  // (the LDS reads after the last stage's barrier fetch operands of a stage that does not exist and are not
+  // used, so the next pass may overwrite the buffers without another barrier)
+  gemm_epilogue<FM, 1, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, blk_off + blk_rows, pid_n * BN + nw * NFW * FM,
+                                         pid_n * BN + BN <= N, 0, lr, h);
+  }  // passes
+  }  // rounds
+}
+
 template <int MR>
 int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
   GemmParams q = p;
@@ -1157,6 +1389,32 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   };
   if (swiglu) return launch(moe_gemm_mxn_kernel<BLKM, MFW, NFW, G, WD, XD, true>);
   return launch(moe_gemm_mxn_kernel<BLKM, MFW, NFW, G, WD, XD, false>);
+}
+
+template <int BLKM, int MFW, int NFW, int WD, int XD>
+int32_t launch_f8n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
+  constexpr int LDS_BYTES = 2 * MFW * 32 * (128 + 16);
+  GemmParams q = p;
+  q.grid_n = (int)cdiv(p.N, 128 * NFW);
+  int64_t grid = (int64_t)grid_m * q.grid_n;
+  if (grid <= 0) return TK_OK;
+  if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
+  q.total_tiles = (int32_t)grid;
+  // persistent grid, one workgroup per CU (the register ring and the accumulators take a wave's whole budget)
+  const int64_t resident = (int64_t)device_cu_count();
+  if (grid > resident) grid = resident;
+  auto launch = [&](auto kern) -> int32_t {
+    static bool attr_done = false;
+    if (!attr_done && LDS_BYTES > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
+      attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
+    return check_launch("moe_gemm_f8n_kernel");
+  };
+  if (swiglu) return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, WD, XD, true>);
+  return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, WD, XD, false>);
 }
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
@@ -1284,6 +1542,19 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.grid_n = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
+  if (d->w_layout == TK_W_TILED && d->w_dtype == TK_E4M3) {
+    if (d->w_mx_scale) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: MX scales with e4m3 weights");
+    if (d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: tiled e4m3 weights take block_m 128 or 256 (got %d)", d->block_m);
+    if (d->K < 16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: K must be at least 16 (got %d)", d->K);
+    if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
+    const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
+    if (d->n_slices > 1 && d->w_stride_e < nfr * nst * 4096) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
+    p.w_stride_e = d->w_stride_e;
+    p.w_nst = (int32_t)nst;
+    //                                          BLKM MFW NFW WD XD
+    if (d->block_m == 256) return launch_f8n<256, 4, 2, 4, 1>(p, d->grid_m, swiglu, st);
+    return launch_f8n<128, 4, 2, 4, 1>(p, d->grid_m, swiglu, st);
+  }
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
     if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);

@@ -31,7 +31,7 @@ from .numerics import InFlexData, OutFlexData
 from .specialize import FnSpecs
 from .tensor import FP4, RaggedTensorMetadata, Tensor, convert_layout, torch_dtype_to_dtype, wrap_torch_tensor
 from .tensor_details.layout_details.cdna4_scale import CDNA4MXScaleLayout
-from .tensor_details.layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
+from .tensor_details.layout_details.gfx950_mx import GFX950FP8ValueLayout, GFX950MXScaleLayout, GFX950MXValueLayout
 from .tensor_details.layout_details.strided import StridedLayout
 
 MXFP_BLOCK_SIZE = 32
@@ -208,7 +208,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if not isinstance(b, Tensor):
         b = wrap_torch_tensor(b, dtype=FP4 if b.dtype == torch.uint8 else None)
     tiled = isinstance(b.storage.layout, GFX950MXValueLayout)
-    if not tiled and not isinstance(b.storage.layout, StridedLayout):
+    tiled_fp8 = isinstance(b.storage.layout, GFX950FP8ValueLayout)
+    if not tiled and not tiled_fp8 and not isinstance(b.storage.layout, StridedLayout):
         raise NotImplementedError(f"weight layout {type(b.storage.layout).__name__} is not supported")
     if b_scale is not None and not isinstance(b_scale, Tensor):
         b_scale = wrap_torch_tensor(b_scale)
@@ -230,7 +231,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         assert precision_config.b_microblock_size is None or precision_config.b_microblock_size == MXFP_BLOCK_SIZE, \
             f"Unsupported microscale block size {precision_config.b_microblock_size}"
     w = b.storage.data
-    if w.ndim == 2 and not tiled:
+    if w.ndim == 2 and not tiled and not tiled_fp8:
         w = w[None]
     K_W, N = b.shape[-2:]
     M = a.shape[-2] if gather_indx is None else gather_indx.shape[0]
@@ -280,7 +281,15 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         assert a_ts.numel() == a.shape[0], "a_mx_tensor_scale must hold one scale per row of a"
         d.x_row_scale = a_ts.data_ptr()
     keep = [a_ts]
-    if tiled:
+    if tiled_fp8:
+        if b_scale is not None:
+            raise NotImplementedError("MX scales are supported with mxfp4 (uint8) weights only")
+        if a.dtype != torch.float8_e4m3fn:
+            raise NotImplementedError("tiled e4m3 weights take e4m3 activations (quantise with quantize_fp8_rowwise)")
+        assert w.is_contiguous() and w.dtype == torch.uint8
+        d.w_dtype = nt.TK_E4M3
+        d.w_layout = nt.TK_W_TILED
+    elif tiled:
         assert b.dtype == FP4 and b_scale is not None, "tiled weights are MXFP4 and need precision_config.b_mx_scale"
         ws = b_scale.storage.data
         assert w.is_contiguous() and ws.is_contiguous() and ws.shape[0] == w.shape[0]
@@ -307,7 +316,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         w = _k_contiguous(w)
         d.w_dtype = nt.TORCH_TO_TK.get(w.dtype, -1)
     d.w = w.data_ptr()
-    if tiled:
+    if tiled or tiled_fp8:
         d.w_stride_e = w.stride(0)
     else:
         d.w_stride_e, d.w_stride_k, d.w_stride_n = w.stride()
@@ -342,7 +351,9 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         d.gammas_dtype = nt.TORCH_TO_TK[g.dtype]
         keep.append(g)
     block_m = opt_flags.block_m
-    if tiled:
+    if tiled_fp8:
+        block_m = 256 if block_m == 256 else 128  # the FP8 MFMA kernel's row blocks
+    elif tiled:
         from .matmul_details.opt_flags import _get_opt_flags_constraints
         if block_m == 128 and _get_opt_flags_constraints().get("block_m") is None and is_ragged and M <= 144 * n_slices:
             block_m = 256  # about 128 rows per expert: one tile per expert, the weights are read once

@@ -9,10 +9,16 @@ that goes with the weight values' layout.
 """
 from .layout_details.base import Layout
 from .layout_details.cdna4_scale import CDNA4MXScaleLayout
-from .layout_details.gfx950_mx import GFX950MXScaleLayout, GFX950MXValueLayout
+from .layout_details.gfx950_mx import GFX950FP8ValueLayout, GFX950MXScaleLayout, GFX950MXValueLayout
 from .layout_details.strided import StridedLayout
 
-__all__ = ["Layout", "StridedLayout", "GFX950MXValueLayout", "GFX950MXScaleLayout", "CDNA4MXScaleLayout"]
+__all__ = ["Layout", "StridedLayout", "GFX950MXValueLayout", "GFX950MXScaleLayout", "GFX950FP8ValueLayout", "CDNA4MXScaleLayout"]
+
+
+def make_default_matmul_fp8_w_layout():
+    """Layout `matmul` prefers for e4m3 expert weights `[E, K, N]` on this GPU (no counterpart in the reference, which
+    takes plain strided fp8 weights; those stay accepted)."""
+    return GFX950FP8ValueLayout()
 
 
 def make_default_matmul_mxfp4_w_layout(mx_axis: int, **_unused):

@@ -13,6 +13,10 @@ columns (N padded to 32) and per K-stage s of 128 (K padded to 128 with zero wei
   scales  one 128-byte block ordered [c:32][4]: the stage's four e8m0 bytes of column F*32 + c.
 
 Storage is a `[E, bytes]` uint8 tensor for both.
+
+`GFX950FP8ValueLayout` is the same idea for e4m3 weights (one byte per element, no MX scales) feeding the FP8 MFMA
+`v_mfma_f32_32x32x64_f8f6f4`: per (F, s) one 4096-byte block ordered [t:2][half:2][h:2][c:32][16 bytes] with the
+bytes of column F*32 + c for k in [s*128 + t*64 + h*32 + half*16, +16).
 """
 from __future__ import annotations
 
@@ -126,4 +130,53 @@ class GFX950MXScaleLayoutTransformation(LayoutTransformation):
         E, KB, N, nfr, nst = self._dims()
         t = data.view(E, nfr, nst, FRAG_N, 4).permute(0, 2, 4, 1, 3)  # [E, s, 4, F, c]
         out = t.reshape(E, nst * 4, nfr * FRAG_N)[:, :KB, :N].contiguous()
+        return out.view(*self.shape)
+
+
+@dataclass(frozen=True)
+class GFX950FP8ValueLayout(Layout):
+
+    @property
+    def name(self):
+        return "GFX950_FP8_VALUE"
+
+    def make_transformation(self, shape, is_fp4: bool) -> LayoutTransformation:
+        if is_fp4:
+            raise ValueError("GFX950FP8ValueLayout holds one-byte (e4m3) values")
+        return GFX950FP8ValueLayoutTransformation(list(shape), is_fp4)
+
+    def swizzle_block_shape(self, block_shape):
+        return block_shape
+
+
+@dataclass(frozen=True)
+class GFX950FP8ValueLayoutTransformation(LayoutTransformation):
+    """Logical operand `[..., K, N]` of one-byte values; storage `[E, nfr * nst * 4096]` uint8."""
+
+    def _dims(self):
+        *lead, K, N = self.shape
+        E = 1
+        for v in lead:
+            E *= v
+        return E, K, N, _cdiv(N, FRAG_N), _cdiv(K, STAGE_K)
+
+    @property
+    def storage_shape(self) -> list:
+        E, K, N, nfr, nst = self._dims()
+        return [E, nfr * nst * 4096]
+
+    def swizzle_data(self, data):
+        """`data`: canonical `[..., K, N]` with unit stride along N (float8 or uint8 bytes)."""
+        E, K, N, nfr, nst = self._dims()
+        pad = torch.zeros((E, nst * STAGE_K, nfr * FRAG_N), dtype=torch.uint8, device=data.device)
+        pad[:, :K, :N] = data.reshape(E, K, N).view(torch.uint8)
+        # k = s*128 + t*64 + h*32 + half*16 + b ; column = F*32 + c
+        t = pad.view(E, nst, 2, 2, 2, 16, nfr, FRAG_N)  # [E, s, t, h, half, b, F, c]
+        t = t.permute(0, 6, 1, 2, 4, 3, 7, 5)  # [E, F, s, t, half, h, c, b]
+        return t.contiguous().view(E, nfr * nst * 4096)
+
+    def unswizzle_data(self, data):
+        E, K, N, nfr, nst = self._dims()
+        t = data.view(E, nfr, nst, 2, 2, 2, FRAG_N, 16).permute(0, 2, 3, 5, 4, 7, 1, 6)  # [E, s, t, h, half, b, F, c]
+        out = t.reshape(E, nst * STAGE_K, nfr * FRAG_N)[:, :K, :N].contiguous()
         return out.view(*self.shape)
