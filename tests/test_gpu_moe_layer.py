@@ -115,7 +115,8 @@ def test_config3_4_mxfp4_reduced_experts(api, device, T, skew, layout):
     assert_allclose_gate(ref, out, what="layer output", max_bad_frac=1e-4)
 
 
-def test_config5_fp8_reduced(api, device):
+@pytest.mark.parametrize("layout", ["strided", "tiled"])
+def test_config5_fp8_reduced(api, device, layout):
     """Mixtral-style FP8: e4m3 weights with per-output-channel fp32 scales, activations quantised per token.
     PARITY UNPINNED by the reference (no reference test feeds row/column scales with plain fp8); the oracle
     dequantises and runs the pinned GEMM oracle."""
@@ -133,7 +134,14 @@ def test_config5_fp8_reduced(api, device):
     w1q, s1 = qw((E, d, f2))
     w2q, s2 = qw((E, f2 // 2, d))
     dev = device
-    kmajor = lambda w: w.to(dev).transpose(-1, -2).contiguous().transpose(-1, -2)
+    def kmajor(w):  # stride 1 along K; "tiled": converted once to the layout `matmul` prefers for e4m3 weights
+        w = w.to(dev).transpose(-1, -2).contiguous().transpose(-1, -2)
+        if layout == "tiled":
+            from triton_kernels.tensor import convert_layout, wrap_torch_tensor
+            from triton_kernels.tensor_details.layout import make_default_matmul_fp8_w_layout
+            w = convert_layout(wrap_torch_tensor(w), make_default_matmul_fp8_w_layout())
+        return w
+
     pc1 = api.PrecisionConfig(b_mx_tensor_scale=s1.to(dev), out_dtype=torch.bfloat16)
     pc2 = api.PrecisionConfig(b_mx_tensor_scale=s2.to(dev), out_dtype=torch.bfloat16)
     out, rdata, h = _layer(api, dev, x, logits, k, kmajor(w1q), None, kmajor(w2q), None, pc1, pc2, fp8=True)

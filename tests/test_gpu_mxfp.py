@@ -164,3 +164,23 @@ def test_baseline_shape_round_trip(mx, device):
         err = (d[e].float() - w[e].float()).abs().view(K // 32, 32, N)
         step = torch.exp2(s[e].float() - 127)  # [K/32, N]
         assert bool((err <= step[:, None, :]).all())
+
+
+@pytest.mark.parametrize("M, K, view", [(37, 4096, "plain"), (5, 1000, "plain"), (9, 1003, "plain"), (6, 520, "offset"), (3, 7, "plain"),
+                                        (4, 14336, "plain")])
+def test_quantize_fp8_rowwise_bit_exact(device, M, K, view):
+    """Per-row e4m3 quantiser (the FP8 configuration's activation path): bytes bit-exact and scales equal to the
+    oracle's, on rows that take the vector path, rows with a scalar tail, and rows that are not 16-byte aligned;
+    one row is all zero (scale 1) and one holds the value that must saturate to 448."""
+    from oracle import moe as omoe
+    from triton_amd.numerics_details.rowwise_fp8 import quantize_fp8_rowwise
+    g = torch.Generator().manual_seed(M * 1000 + K)
+    base = (torch.randn((M, K + 8), generator=g) * 3).to(torch.bfloat16)
+    base[0] = 0
+    x = base[:, 1:K + 1] if view == "offset" else base[:, :K]
+    xd = base.to(device)
+    xd = xd[:, 1:K + 1] if view == "offset" else xd[:, :K]
+    q, s = quantize_fp8_rowwise(xd)
+    q_ref, s_ref = omoe.quantize_fp8_rowwise(x)
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))

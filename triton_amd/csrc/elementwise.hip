@@ -87,22 +87,43 @@ __global__ __launch_bounds__(256) void reduce_mid_bf16x8_kernel(const uint16_t* 
 }
 
 // Per-row dynamic quantisation to OCP e4m3: s = amax / 448 (1 for an all-zero row), q = sat(x / s).
-// One wave per row; the row is read twice (second pass hits L2).
+// One wave per row; the row is read twice (second pass hits L2), 16 bytes per lane and load where aligned.
 __global__ __launch_bounds__(256) void quant_fp8_rows_kernel(const uint16_t* x, int64_t stride_m, int64_t M, int64_t K,
                                                              uint8_t* q, int64_t stride_qm, float* scales) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= M) return;
   const uint16_t* xr = x + row * stride_m;
+  uint8_t* qr = q + row * stride_qm;
+  // 16-byte loads / 8-byte stores when rows allow it (the scalar loop covers the rest of the row, or all of it)
+  const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15) | (reinterpret_cast<uintptr_t>(qr) & 7)) == 0;
+  const int64_t kv = vec ? (K & ~int64_t(7)) : 0;
   float m = 0.f;
-  for (int64_t k = lane; k < K; k += 64) m = fmaxf(m, fabsf(bf16_bits_to_f32(xr[k])));
+  for (int64_t k = lane * 8; k < kv; k += 512) {
+    const uint4 v = *reinterpret_cast<const uint4*>(xr + k);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) m = fmaxf(m, fmaxf(fabsf(bits_f32(w[i] << 16)), fabsf(bits_f32(w[i] & 0xFFFF0000u))));
+  }
+  for (int64_t k = kv + lane; k < K; k += 64) m = fmaxf(m, fabsf(bf16_bits_to_f32(xr[k])));
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   float s = m / 448.0f;
   if (s == 0.f) s = 1.0f;
   if (lane == 0) scales[row] = s;
-  uint8_t* qr = q + row * stride_qm;
-  for (int64_t k = lane; k < K; k += 64) qr[k] = (uint8_t)e4m3_byte(mx_clamp(bf16_bits_to_f32(xr[k]) / s, 448.0f));
+  for (int64_t k = lane * 8; k < kv; k += 512) {
+    const uint4 v = *reinterpret_cast<const uint4*>(xr + k);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = e4m3_byte(mx_clamp(bits_f32(w[i] << 16) / s, 448.0f));
+      const uint32_t hi = e4m3_byte(mx_clamp(bits_f32(w[i] & 0xFFFF0000u) / s, 448.0f));
+      o[i >> 1] |= ((lo & 0xFFu) | ((hi & 0xFFu) << 8)) << (16 * (i & 1));
+    }
+    *reinterpret_cast<uint2*>(qr + k) = make_uint2(o[0], o[1]);
+  }
+  for (int64_t k = kv + lane; k < K; k += 64) qr[k] = (uint8_t)e4m3_byte(mx_clamp(bf16_bits_to_f32(xr[k]) / s, 448.0f));
 }
 
 int grid_for(int64_t total) {

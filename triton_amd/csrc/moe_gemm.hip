@@ -1126,7 +1126,7 @@ template <int BLKM, int MFW, int NFW, int WD, int XD, bool SWIGLU>
 __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   typedef Frag<32> FR;
   constexpr int FM = 32, BM = MFW * 32, BN = 128 * NFW, KC = 128;
-  static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2), "ring depths");
+  static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2 || XD == 4) && WD % XD == 0, "ring depths");
   constexpr int XPITCH = KC + 16;
   constexpr int XBYTES = BM * XPITCH;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -1287,20 +1287,18 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1 % XD); });
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (WD == 4) {
-      load_w(S1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (XD == 2) {
-      static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 2, 0); });
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (WD == 4) {
-      load_w(S2, 2);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    // activations of stages 1..XD and weights of stages 1..WD-2, alternating, oldest first
+    static_for<1, (XD > WD - 2 ? XD : WD - 2) + 1>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i <= XD) {
+        static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, i, i % XD); });
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (i <= WD - 2) {
+        load_w(template_int<i>{}, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
