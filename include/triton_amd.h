@@ -177,7 +177,8 @@ int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t
  *   scales  one 128-byte block at ((F * S + s) * 128) ordered [c:32][4]: the four e8m0 bytes of column
  *           F*32 + c for the stage's four 32-element blocks.
  * With w_dtype == TK_E4M3 (e4m3 activations, no MX scales) TK_W_TILED is the one-byte variant of the same idea:
- *   values  one 4096-byte block at ((F * S + s) * 4096) ordered [q:4][lane:64][16 bytes]; lane = h*32 + c holds
+ *   values  K padded to 256 (S = 2 * ceil(K / 256) blocks of 128 per fragment); one 4096-byte block at
+ *           ((F * S + s) * 4096) ordered [q:4][lane:64][16 bytes]; lane = h*32 + c holds
  *           the e4m3 bytes of column F*32 + c for k in [s*128 + (q/2)*64 + h*32 + (q%2)*16, +16);
  *           block_m must be 128 or 256.
  * The w_stride_e / ws_stride_e fields give the bytes from one expert to the next; the k / n strides are unused.

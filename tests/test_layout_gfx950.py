@@ -63,7 +63,7 @@ def test_fp8_value_layout_round_trip_and_placement(E, K, N):
     t = wrap_torch_tensor(w)
     assert t.shape == [E, K, N]
     tiled = convert_layout(t, GFX950FP8ValueLayout())
-    nfr, nst = (N + 31) // 32, (K + 127) // 128
+    nfr, nst = (N + 31) // 32, 2 * ((K + 255) // 256)
     assert list(tiled.storage.data.shape) == [E, nfr * nst * 4096] == GFX950FP8ValueLayout().storage_shape([E, K, N], False)
     back = convert_layout(tiled, StridedLayout(-2))
     assert torch.equal(back.storage.data.view(torch.uint8), w.view(torch.uint8))

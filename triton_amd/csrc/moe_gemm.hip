@@ -1108,27 +1108,30 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
 // e4m3 weights in a tile-native layout x e4m3 activations (prefill): FP8 MFMA, no conversion in the loop
 // ------------------------------------------------------------------------------------------------
 // Weight layout (built once per model by the host from the K-contiguous form): per expert, per fragment F of 32
-// output columns (N padded to 32), per K-stage s of 128 (K padded to 128 with zero weights): one 4 KiB block
-// [q:4][lane:64][16 B]; lane = h*32 + lr holds the e4m3 bytes of column F*32 + lr for
-// k in [s*128 + (q/2)*64 + h*32 + (q%2)*16, +16): pieces 2t and 2t+1 of a lane are the 32 consecutive bytes it
-// feeds to the v_mfma_f32_32x32x64_f8f6f4 of K-step t.  The activation rows (gathered, one byte per element)
-// are staged through LDS with a 144-byte row pitch and read back as the same 32 consecutive bytes per lane, so
-// both operands put the same k in the same byte position whatever order the instruction sums them in.
-// Per-row and per-column fp32 scales, bias, activation and gate weight are applied by the shared epilogue.
+// output columns (N padded to 32), per K-block s of 128 (K padded to 256 with zero weights, so the number of
+// blocks is even): one 4 KiB block [q:4][lane:64][16 B]; lane = h*32 + lr holds the e4m3 bytes of column
+// F*32 + lr for k in [s*128 + (q/2)*64 + h*32 + (q%2)*16, +16): pieces 2t and 2t+1 of a lane are the 32 consecutive
+// bytes it feeds to the v_mfma_f32_32x32x64_f8f6f4 of K-step t.  The activation rows (gathered, one byte per
+// element) are staged through LDS and read back as the same 32 consecutive bytes per lane, so both operands put
+// the same k in the same byte position whatever order the instruction sums them in.  Per-row and per-column
+// fp32 scales, bias, activation and gate weight are applied by the shared epilogue.
 //
 // Structure as in the MXFP4 prefill kernel: four waves, each owning NFW column fragments whose weights go
-// global memory -> register ring (WD stages deep) -> MFMA, all sharing the MFW row fragments of the tile through
-// an LDS double buffer; two K-steps per stage; one workgroup barrier per stage, in step 1; persistent grid with
-// XCD-aware rounds and (expert, column tile, row block) tile order.
+// global memory -> register double buffer -> MFMA, all sharing the MFW row fragments of the tile through an LDS
+// double buffer; persistent grid with XCD-aware rounds and (expert, column tile, row block) tile order.  A stage
+// is 256 bytes of K = four K-steps of 64, one workgroup barrier per stage (in step 3); the 64 memory instructions
+// of a stage (LDS reads of the next step's activations, LDS writes of the next stage's activations with the
+// refill of their staging registers, weight loads of the next stage) are dealt two or three to each of the 32
+// MFMA slots: a slot that issues many loads back to back holds up the next MFMA.
 typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
 
-template <int BLKM, int MFW, int NFW, int WD, int XD, bool SWIGLU>
+template <int BLKM, int MFW, int NFW, bool SWIGLU>
 __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   typedef Frag<32> FR;
-  constexpr int FM = 32, BM = MFW * 32, BN = 128 * NFW, KC = 128;
-  static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2 || XD == 4) && WD % XD == 0, "ring depths");
+  constexpr int FM = 32, BM = MFW * 32, BN = 128 * NFW, KC = 256, NS = 4;
   constexpr int XPITCH = KC + 16;
   constexpr int XBYTES = BM * XPITCH;
+  constexpr int XCH = 2 * MFW;  // 16-byte activation pieces per thread per stage
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int tid = threadIdx.x;
@@ -1136,7 +1139,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   const int nw = __builtin_amdgcn_readfirstlane(tid >> 6);  // column quarter of the tile
   const int lr = lane & 31, h = lane >> 5;
   const int K = p.K, N = p.N;
-  const int nst = p.w_nst;
+  const int nst = p.w_nst;  // stages of 256 (two 4 KiB weight blocks per column fragment each)
   const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
   for (int round0 = 0; round0 < live; round0 += (int)gridDim.x) {
   const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
@@ -1165,17 +1168,17 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   const int rows = (blk_rows - pass_off) < BM ? (blk_rows - pass_off) : BM;
   const int nj = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW)
 
-  // ---- activation staging: piece j of this thread = row 32 j + tid/8, 16-byte chunk tid%8 of the stage ----
-  const int xc = tid & 7;
-  const uint8_t* xptr[MFW];
+  // ---- activation staging: piece j of this thread = row 16 j + tid/16, 16-byte chunk tid%16 of the stage ----
+  const int xc = tid & 15;
+  const uint8_t* xptr[XCH];
 #pragma unroll
-  for (int j = 0; j < MFW; ++j) {
-    int row = off_m + (tid >> 3) + 32 * j;
+  for (int j = 0; j < XCH; ++j) {
+    int row = off_m + (tid >> 4) + 16 * j;
     row = row < eM ? row : eM - 1;
     const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
     xptr[j] = p.x + src * p.x_stride_m;
   }
-  const int xlds0 = (tid >> 3) * XPITCH + xc * 16;  // piece j at xlds0 + j*32*XPITCH
+  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // piece j at xlds0 + j*16*XPITCH
 
   const int nfr = (N + 31) >> 5;
   const uint8_t* wptr[NFW];
@@ -1183,7 +1186,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   for (int f = 0; f < NFW; ++f) {
     int F = pid_n * (BN / 32) + nw * NFW + f;
     F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
-    wptr[f] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 4096 + lane * 16;
+    wptr[f] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 8192 + lane * 16;
   }
 
   typename FR::acc_t acc[NFW][MFW];
@@ -1194,31 +1197,28 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
 #pragma unroll
       for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
 
-  u32x4_t xreg[XD][MFW];
-  i32x8_t wreg[WD][NFW][2];  // [ring slot][column fragment][K-step]
-  i32x8_t xf[2][MFW];        // [K-step][row fragment]
+  u32x4_t xreg[XCH];
+  i32x8_t wreg[2][NFW][NS];  // [stage parity][column fragment][K-step]
+  i32x8_t xf[2][MFW];        // [K-step parity][row fragment]
 
   // Loads are unconditional: rows past the last valid row re-read it, k past K re-reads the row's last 16 bytes
   // (the padded weights there are zero), stages past the last one re-read the last stage.
-  auto load_x_piece = [&](int j, int s, int slot) __attribute__((always_inline)) {
+  auto load_x_piece = [&](int j, int s) __attribute__((always_inline)) {
     int k0 = s * KC + xc * 16;
     k0 = k0 < K - 16 ? k0 : K - 16;
-    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0);
+    xreg[j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0);
   };
-  auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
-    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 32 * XPITCH) = xreg[slot][j];
+  auto store_x_piece = [&](int j, int buf) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 16 * XPITCH) = xreg[j];
   };
-  auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
+  // weights of K-step t of column fragment f, stage s, into register set SL
+  auto load_w = [&](auto slot_c, int f, int t, int s) __attribute__((always_inline)) {
     constexpr int SL = decltype(slot_c)::value;
     s = s < nst ? s : nst - 1;
-#pragma unroll
-    for (int f = 0; f < NFW; ++f)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 4096 + (2 * t) * 1024);
-        const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 4096 + (2 * t + 1) * 1024);
-        wreg[SL][f][t] = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
+    const uint8_t* a = wptr[f] + (int64_t)s * 8192 + t * 2048;
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(a);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(a + 1024);
+    wreg[SL][f][t] = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
   auto read_xf = [&](int buf, int t, int j, i32x8_t (&out)[MFW]) __attribute__((always_inline)) {
     const uint8_t* a = lds + buf * XBYTES + (j * FM + lr) * XPITCH + t * 64 + h * 32;
@@ -1229,44 +1229,48 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
 
   template_int<0> S0;
   template_int<1> S1;
-  template_int<2> S2;
-  template_int<3> S3;
 
-  // One K-stage (two K-steps of 64).  NJ = row fragments with valid rows; WS = c % WD = weight ring slot, the LDS
-  // buffer is WS & 1.  Step 0 interleaves, between its MFMAs: the LDS reads of step 1's activations, the LDS
-  // writes of the next stage's activations (other buffer) with the refill of their staging registers, and the
-  // weight loads WD-1 stages ahead.  Step 1: after its first MFMA every wave has read all it needs from this
-  // stage's buffer and written its share of the next one; barrier; then the reads of the next stage's step 0.
-  auto stage = [&](auto nj_c, auto ws_c, int c) __attribute__((always_inline)) {
+  // One stage.  NJ = row fragments with valid rows; PAR = c & 1 = LDS buffer and weight register set.
+  // Ops of step t: NJ reads of step t+1's activation fragments (step 3: the next stage's step 0, after the
+  // barrier), in steps 0..2 the staging of the next stage's activations (2 NJ pieces over three steps) and in
+  // every step two (fragment, K-step) pairs of the next stage's weights.
+  auto stage = [&](auto nj_c, auto par_c, int c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    constexpr int WS = decltype(ws_c)::value;
-    constexpr int PAR = WS & 1;
-    using WSL = template_int<(WS + WD - 1) % WD>;
-    constexpr int XS = (WS + 1) % XD;
+    constexpr int PAR = decltype(par_c)::value;
+    using NXT = template_int<PAR ^ 1>;
     constexpr int NM = NJ * NFW;
-    constexpr int NOPS = 2 * NJ + 1;
-    static_for<0, 2>([&](auto t_c) __attribute__((always_inline)) {
+    constexpr int NP = 2 * NJ;
+    constexpr int PPS = (NP + 2) / 3;          // pieces staged per step during steps 0..2
+    constexpr int WPS = (NFW * NS + NS - 1) / NS;  // weight (fragment, K-step) pairs loaded per step
+    constexpr int NOPS = NJ + PPS + WPS;
+    static_for<0, NS>([&](auto t_c) __attribute__((always_inline)) {
       constexpr int t = decltype(t_c)::value;
+      constexpr int cur = t & 1, nxt = cur ^ 1;
       auto op = [&](auto o_c) __attribute__((always_inline)) {
         constexpr int o = decltype(o_c)::value;
-        if constexpr (t == 0) {
-          if constexpr (o < NJ) {
-            read_xf(PAR, 1, o, xf[1]);
-          } else if constexpr (o < 2 * NJ) {
-            store_x_piece(o - NJ, PAR ^ 1, XS);
-            load_x_piece(o - NJ, c + 1 + XD, XS);
-          } else {
-            load_w(WSL{}, c + WD - 1);
+        if constexpr (o < NJ) {
+          if constexpr (t < NS - 1)
+            read_xf(PAR, t + 1, o, xf[nxt]);
+          else
+            read_xf(PAR ^ 1, 0, o, xf[nxt]);
+        } else if constexpr (o < NJ + PPS) {
+          constexpr int j = t * PPS + (o - NJ);
+          if constexpr (t < NS - 1 && j < NP) {
+            store_x_piece(j, PAR ^ 1);
+            load_x_piece(j, c + 2);
           }
         } else {
-          if constexpr (o < NJ) read_xf(PAR ^ 1, 0, o, xf[0]);
+          constexpr int w = t * WPS + (o - NJ - PPS);
+          if constexpr (w < NFW * NS) load_w(NXT{}, w % NFW, w / NFW, c + 1);  // in the order the K-steps use them
         }
       };
       static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
         constexpr int m = decltype(m_c)::value;
         constexpr int j = m / NFW, f = m % NFW;
-        acc[f][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wreg[WS][f][t], xf[t][j], acc[f][j], 0, 0, 0, 0, 0, 0);
-        if constexpr (t == 1 && m == 0) {
+        acc[f][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wreg[PAR][f][t], xf[cur][j], acc[f][j], 0, 0, 0, 0, 0, 0);
+        if constexpr (t == NS - 1 && m == 0) {
+          // every wave has fetched its last operands of this buffer (during step 2) and written its share of
+          // the next one (steps 0..2)
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
           __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -1279,49 +1283,30 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
 
   auto run = [&](auto nj_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    // Prologue: stage 0 without overlap; the loads left in flight are issued in the order the steady state leaves
-    // them in at the top of a stage (activations, then weights, of stage 1, then of stage 2).
-    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
+    constexpr int NP = 2 * NJ;
+    // Prologue: stage 0 without overlap; the loads left in flight (activations, then weights, of stage 1) are
+    // issued in the order the steady state leaves them in at the top of a stage.
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    load_w(S0, 0);
+    static_for<0, NFW * NS>([&](auto wc) __attribute__((always_inline)) { load_w(S0, decltype(wc)::value % NFW, decltype(wc)::value / NFW, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0); });
     __builtin_amdgcn_sched_barrier(0);
-    // activations of stages 1..XD and weights of stages 1..WD-2, alternating, oldest first
-    static_for<1, (XD > WD - 2 ? XD : WD - 2) + 1>([&](auto ic) __attribute__((always_inline)) {
-      constexpr int i = decltype(ic)::value;
-      if constexpr (i <= XD) {
-        static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, i, i % XD); });
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if constexpr (i <= WD - 2) {
-        load_w(template_int<i>{}, i);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    });
+    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1); });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NFW * NS>([&](auto wc) __attribute__((always_inline)) { load_w(S1, decltype(wc)::value % NFW, decltype(wc)::value / NFW, 1); });
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { read_xf(0, 0, decltype(jc)::value, xf[0]); });
     __builtin_amdgcn_sched_barrier(0);
     int c = 0;
-    if constexpr (WD == 4) {
-      for (; c + 3 < nst; c += 4) {
-        stage(nj_c, S0, c);
-        stage(nj_c, S1, c + 1);
-        stage(nj_c, S2, c + 2);
-        stage(nj_c, S3, c + 3);
-      }
-      if (c < nst) stage(nj_c, S0, c);
-      if (c + 1 < nst) stage(nj_c, S1, c + 1);
-      if (c + 2 < nst) stage(nj_c, S2, c + 2);
-    } else {
-      for (; c + 1 < nst; c += 2) {
-        stage(nj_c, S0, c);
-        stage(nj_c, S1, c + 1);
-      }
-      if (c < nst) stage(nj_c, S0, c);
+    for (; c + 1 < nst; c += 2) {
+      stage(nj_c, S0, c);
+      stage(nj_c, S1, c + 1);
     }
+    if (c < nst) stage(nj_c, S0, c);
   };
   static_for<1, MFW + 1>([&](auto n_c) __attribute__((always_inline)) {
     if (nj == decltype(n_c)::value) run(n_c);
@@ -1389,9 +1374,9 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   return launch(moe_gemm_mxn_kernel<BLKM, MFW, NFW, G, WD, XD, false>);
 }
 
-template <int BLKM, int MFW, int NFW, int WD, int XD>
+template <int BLKM, int MFW, int NFW>
 int32_t launch_f8n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
-  constexpr int LDS_BYTES = 2 * MFW * 32 * (128 + 16);
+  constexpr int LDS_BYTES = 2 * MFW * 32 * (256 + 16);
   GemmParams q = p;
   q.grid_n = (int)cdiv(p.N, 128 * NFW);
   int64_t grid = (int64_t)grid_m * q.grid_n;
@@ -1411,8 +1396,8 @@ int32_t launch_f8n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
     return check_launch("moe_gemm_f8n_kernel");
   };
-  if (swiglu) return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, WD, XD, true>);
-  return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, WD, XD, false>);
+  if (swiglu) return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, true>);
+  return launch(moe_gemm_f8n_kernel<BLKM, MFW, NFW, false>);
 }
 
 template <int WK, int FM, int WM, int WN, int MFW, int NFW, int KS>
@@ -1545,13 +1530,13 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: tiled e4m3 weights take block_m 128 or 256 (got %d)", d->block_m);
     if (d->K < 16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: K must be at least 16 (got %d)", d->K);
     if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
-    const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
-    if (d->n_slices > 1 && d->w_stride_e < nfr * nst * 4096) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
+    const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 256);  // stages of 256 = two 4 KiB blocks per fragment
+    if (d->n_slices > 1 && d->w_stride_e < nfr * nst * 8192) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
-    //                                          BLKM MFW NFW WD XD
-    if (d->block_m == 256) return launch_f8n<256, 4, 2, 4, 1>(p, d->grid_m, swiglu, st);
-    return launch_f8n<128, 4, 2, 4, 1>(p, d->grid_m, swiglu, st);
+    //                                          BLKM MFW NFW
+    if (d->block_m == 256) return launch_f8n<256, 4, 2>(p, d->grid_m, swiglu, st);
+    return launch_f8n<128, 4, 2>(p, d->grid_m, swiglu, st);
   }
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");

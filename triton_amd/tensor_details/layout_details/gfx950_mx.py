@@ -15,7 +15,7 @@ columns (N padded to 32) and per K-stage s of 128 (K padded to 128 with zero wei
 Storage is a `[E, bytes]` uint8 tensor for both.
 
 `GFX950FP8ValueLayout` is the same idea for e4m3 weights (one byte per element, no MX scales) feeding the FP8 MFMA
-`v_mfma_f32_32x32x64_f8f6f4`: per (F, s) one 4096-byte block ordered [t:2][half:2][h:2][c:32][16 bytes] with the
+`v_mfma_f32_32x32x64_f8f6f4`: K is padded to 256 (an even number of 128-blocks) and per (F, s) one 4096-byte block ordered [t:2][half:2][h:2][c:32][16 bytes] with the
 bytes of column F*32 + c for k in [s*128 + t*64 + h*32 + half*16, +16).
 """
 from __future__ import annotations
@@ -158,7 +158,7 @@ class GFX950FP8ValueLayoutTransformation(LayoutTransformation):
         E = 1
         for v in lead:
             E *= v
-        return E, K, N, _cdiv(N, FRAG_N), _cdiv(K, STAGE_K)
+        return E, K, N, _cdiv(N, FRAG_N), 2 * _cdiv(K, 2 * STAGE_K)  # K padded to 256: an even number of 128-blocks
 
     @property
     def storage_shape(self) -> list:
