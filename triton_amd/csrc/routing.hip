@@ -413,7 +413,17 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
   for (int e = threadIdx.x; e < E; e += kScanThreads) hist_s[e] = 0;
   for (int f = threadIdx.x; f < R; f += kScanThreads) eid_s[f] = -1;
   __syncthreads();
-  // ---- phase 1: top-k per row (wave w takes rows w, w + 16, ...) ----
+  // ---- phase 1: top-k per row (wave w takes rows w, w + 16, ...); the next row's logits are fetched while the
+  // current row is selected, so a wave pays the memory latency once ----
+  float nv[EPL];
+  auto load_row = [&](int row) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      nv[i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
+    }
+  };
+  if (!p.use_provided_indx && wave < T && wave < n_rows) load_row(wave);
   for (int row = wave; row < T && row < n_rows; row += kScanWaves) {
     float myval = 0.f;
     int myidx = -1;
@@ -427,12 +437,10 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
 #pragma unroll
       for (int i = 0; i < EPL; ++i) {
         const int e = lane + 64 * i;
-        key[i] = 0ull;
-        if (e < E) {
-          const float v = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e);
-          key[i] = ((unsigned long long)ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e);
-        }
+        key[i] = e < E ? ((unsigned long long)ordered_key(nv[i]) << 32) | (uint32_t)(~(uint32_t)e) : 0ull;
       }
+      const int nrow = row + kScanWaves;
+      if (nrow < T && nrow < n_rows) load_row(nrow);
       for (int j = 0; j < k; ++j) {
         unsigned long long best = key[0];
 #pragma unroll
