@@ -89,6 +89,10 @@ CASES = [
     ((2, 16, 512), -1, torch.float8_e4m3fn, 1),
     ((5, 96, 33), 1, torch.uint8, 0),  # odd inner: one column per lane
     ((2, 64, 130), 1, torch.float8_e4m3fn, 0),
+    ((3, 96, 516), 1, torch.uint8, 1),  # tile kernels: partial column tile, 3 of 8 blocks
+    ((2, 160, 260), 1, torch.float8_e4m3fn, 0),  # 5 blocks = one full fp8 tile of 4 + 1
+    ((2, 352, 1028), 1, torch.float8_e5m2, 1),
+    ((4, 288, 8, 36), 1, torch.uint8, 0),  # two inner dims
     ((7, 2880), 1, torch.uint8, 0),
     ((2880, 6), 0, torch.uint8, 0),
 ]
@@ -184,3 +188,21 @@ def test_quantize_fp8_rowwise_bit_exact(device, M, K, view):
     q_ref, s_ref = omoe.quantize_fp8_rowwise(x)
     assert torch.equal(s.cpu(), s_ref)
     assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_infinite_inputs_match_oracle(mx, device, dt):
+    """+-inf elements: the block scale becomes 2^128 (byte 255), inf * 0 is NaN and saturates to +-6 with the sign of its
+    bit pattern, the finite elements of the block become 0 (mxfp.py:255-327); checked on the strided-axis kernels
+    (LDS-transposed tile path and the plain one) against the oracle.  NaN inputs are left out: whether the block
+    maximum propagates them differs between the reference's own two implementations."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn((2, 64, 260), generator=g).to(dt)
+    x[0, 3, 5] = float("inf")
+    x[0, 40, 7] = float("-inf")
+    x[1, 33, 259] = float("-inf")
+    for xs in (x, x[:, :, :131].contiguous()):  # inner 260: tile kernels; inner 131: one column per lane
+        q, s = mx.downcast_to_mxfp(xs.to(device), torch.uint8, axis=1)
+        qo, so = omx.downcast_to_mxfp(xs, torch.uint8, axis=1)
+        _same(qo, q, "values")
+        _same(so, s, "scales")

@@ -256,6 +256,219 @@ __global__ __launch_bounds__(kThreads) void mx_up_cols(const uint8_t* __restrict
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// 16-bit sources / destinations with the inner axis contiguous, through an LDS transpose.
+// A workgroup takes 256 columns x NB blocks of 32 rows, NB chosen so that the NB blocks of one column are
+// 128 output bytes (8 blocks of e2m1, 4 of fp8): the quantised bytes of a column are then moved as one full
+// 128-byte line (8 lanes x 16 bytes) instead of 16- or 32-byte pieces of 64 different lines per instruction,
+// and a lane walks its rows with 8-byte accesses (4 columns), so a wave covers 512 contiguous bytes per row.
+// ---------------------------------------------------------------------------------------------
+constexpr int kTileCols = 256;
+constexpr int kTilePitch = 128 + 16;  // LDS bytes per column
+// LDS row of tile column c: a lane's four adjacent columns are spread 65 rows apart, so the 16-byte accesses of
+// consecutive lanes (columns c, c + 4, ...) fall 144 bytes apart and take different banks
+constexpr int kTileRows = 64 + 65 * 3;
+__device__ __forceinline__ int tile_row(int c) { return (c >> 2) + 65 * (c & 3); }
+
+template <int KIND>
+struct TileGeom {
+  static constexpr int BB = KIND == TK_E2M1 ? 16 : 32;  // value bytes per block and column
+  static constexpr int NB = 128 / BB;                    // blocks per tile
+};
+
+// moves the tile's value bytes and scales between LDS and global memory (TO_GLOBAL) or back
+template <int KIND, bool TO_GLOBAL>
+__device__ __forceinline__ void tile_move(uint8_t* vals_s, uint8_t* sc_s, uint8_t* gvals, uint8_t* gscales, int64_t o, int64_t col0,
+                                          int64_t blk0, int64_t L, int64_t inner, int64_t inner_last) {
+  constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
+  const int64_t nblk = L / 32;
+  const int64_t line_bytes = KIND == TK_E2M1 ? L / 2 : L;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int q = it * kThreads + threadIdx.x;
+    const int col = q >> 3, piece = q & 7;
+    const int64_t blk = blk0 + piece * 16 / BB;
+    if (col0 + col < inner && blk < nblk) {
+      const int64_t line = line_of(o, col0 + col, inner, inner_last);
+      uint4* g = reinterpret_cast<uint4*>(gvals + line * line_bytes + blk0 * BB + piece * 16);
+      uint4* l = reinterpret_cast<uint4*>(vals_s + tile_row(col) * kTilePitch + piece * 16);
+      if (TO_GLOBAL)
+        *g = *l;
+      else
+        *l = *g;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NB; ++it) {
+    const int q = it * kThreads + threadIdx.x;
+    const int col = q / NB, b = q % NB;
+    if (col0 + col < inner && blk0 + b < nblk) {
+      const int64_t line = line_of(o, col0 + col, inner, inner_last);
+      if (TO_GLOBAL)
+        gscales[line * nblk + blk0 + b] = sc_s[col * NB + b];
+      else
+        sc_s[col * NB + b] = gscales[line * nblk + blk0 + b];
+    }
+  }
+}
+
+template <int SRC, int KIND>
+__global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restrict__ src, int64_t stride_outer, int64_t stride_axis,
+                                                         int64_t L, int64_t inner, int64_t inner_last, int64_t col_tiles,
+                                                         int64_t blk_tiles, uint8_t* __restrict__ out_vals,
+                                                         uint8_t* __restrict__ out_scales, int rounding) {
+  constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
+  __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
+  __shared__ uint8_t sc_s[kTileCols * NB];
+  int64_t bid = blockIdx.x;
+  const int64_t ct = bid % col_tiles;
+  bid /= col_tiles;
+  const int64_t bt = bid % blk_tiles;
+  const int64_t o = bid / blk_tiles;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
+  const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
+  const int c4 = lane * 4;  // this lane's four columns inside the tile
+#pragma unroll 1
+  for (int pass = 0; pass < NB / 4; ++pass) {
+    const int b = wave + 4 * pass;
+    if (blk0 + b >= L / 32 || col0 + c4 >= inner) continue;
+    const uint16_t* p = src + o * stride_outer + (blk0 + b) * 32 * stride_axis + col0 + c4;
+    // the 32 rows stay packed (two 16-bit elements per register) and are widened where they are used: half the
+    // registers of an fp32 copy, which is what lets four workgroups share a CU and overlap their load phases
+    uint2 raw[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) raw[i] = *reinterpret_cast<const uint2*>(p + i * stride_axis);
+    auto elem = [&](int i, int c) __attribute__((always_inline)) {
+      const uint32_t w = c < 2 ? raw[i].x : raw[i].y;
+      const uint16_t e = (uint16_t)((c & 1) ? (w >> 16) : (w & 0xFFFFu));
+      return Elem<SRC>::load(&e);
+    };
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float m = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(elem(i, c)));
+      const uint32_t sbits = mx_scale_bits(m, KIND, rounding);
+      const float inv = mx_inv_scale(sbits);
+      uint4* dst = reinterpret_cast<uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
+      if (KIND == TK_E2M1) {
+        // hardware conversion (round to nearest even, saturating at +-6); NaN is first turned into the infinity of
+        // its sign so that it saturates like the reference's bit algorithm (mxfp.py:298-327)
+        uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 32; i += 2) {
+          float q0 = elem(i, c) * inv, q1 = elem(i + 1, c) * inv;
+          q0 = q0 != q0 ? __builtin_copysignf(INFINITY, q0) : q0;
+          q1 = q1 != q1 ? __builtin_copysignf(INFINITY, q1) : q1;
+          if ((i & 6) == 0) w[i >> 3] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w[i >> 3], q0, q1, 1.0f, 0);
+          if ((i & 6) == 2) w[i >> 3] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w[i >> 3], q0, q1, 1.0f, 1);
+          if ((i & 6) == 4) w[i >> 3] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w[i >> 3], q0, q1, 1.0f, 2);
+          if ((i & 6) == 6) w[i >> 3] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w[i >> 3], q0, q1, 1.0f, 3);
+        }
+        dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+      } else {
+        uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 32; ++i) w[i >> 2] |= quant_byte<KIND>(elem(i, c) * inv) << (8 * (i & 3));
+        dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        dst[BB / 32] = make_uint4(w[4], w[5], w[6], w[7]);
+      }
+      sc_s[(c4 + c) * NB + b] = (uint8_t)(sbits >> 23);
+    }
+  }
+  __syncthreads();
+  tile_move<KIND, true>(vals_s, sc_s, out_vals, out_scales, o, col0, blk0, L, inner, inner_last);
+}
+
+template <int KIND, int DST>
+__global__ __launch_bounds__(kThreads) void mx_up_tile(const uint8_t* __restrict__ vals, const uint8_t* __restrict__ scales, int64_t L,
+                                                       int64_t inner, int64_t inner_last, int64_t col_tiles, int64_t blk_tiles,
+                                                       uint16_t* __restrict__ out, int64_t ostride_outer, int64_t ostride_axis) {
+  constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
+  __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
+  __shared__ uint8_t sc_s[kTileCols * NB];
+  int64_t bid = blockIdx.x;
+  const int64_t ct = bid % col_tiles;
+  bid /= col_tiles;
+  const int64_t bt = bid % blk_tiles;
+  const int64_t o = bid / blk_tiles;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
+  const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
+  const int c4 = lane * 4;
+  tile_move<KIND, false>(vals_s, sc_s, const_cast<uint8_t*>(vals), const_cast<uint8_t*>(scales), o, col0, blk0, L, inner, inner_last);
+  __syncthreads();
+  const float mf = Elem<DST>::max_finite();
+#pragma unroll 1
+  for (int pass = 0; pass < NB / 4; ++pass) {
+    const int b = wave + 4 * pass;
+    if (blk0 + b >= L / 32 || col0 + c4 >= inner) continue;
+    uint32_t hp[32][2];  // the lane's four columns of each row as two packed pairs
+    auto put = [&](int i, int c, uint32_t h16) __attribute__((always_inline)) {
+      if (c & 1)
+        hp[i][c >> 1] |= h16 << 16;
+      else
+        hp[i][c >> 1] = h16;
+    };
+    auto put_f = [&](int i, int c, float f) __attribute__((always_inline)) {
+      uint16_t e;
+      Elem<DST>::store(&e, f);
+      put(i, c, e);
+    };
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t sb = sc_s[(c4 + c) * NB + b];
+      const uint4* srcp = reinterpret_cast<const uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
+      if (KIND == TK_E2M1) {
+        const uint4 w4 = srcp[0];
+        const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+        // Hardware conversion where element * scale is a normal number of the target type whatever the element
+        // (then it is exact and needs no clamp); blocks with extreme scales take the bit algorithm.
+        const bool fast = DST == TK_BF16 ? (sb >= 8 && sb <= 248) : (sb >= 114 && sb <= 139);
+        if (fast) {
+          const float scale = hd_bits_f32(sb << 23);
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              uint32_t pr;
+              if (DST == TK_BF16) {
+                bf16x2_t r = g == 0   ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 0)
+                             : g == 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 1)
+                             : g == 2 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 2)
+                                      : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 3);
+                pr = __builtin_bit_cast(uint32_t, r);
+              } else {
+                f16x2_t r = g == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 0)
+                            : g == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 1)
+                            : g == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 2)
+                                     : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 3);
+                pr = __builtin_bit_cast(uint32_t, r);
+              }
+              put(d * 8 + g * 2, c, pr & 0xFFFFu);
+              put(d * 8 + g * 2 + 1, c, pr >> 16);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 32; ++i)
+            put_f(i, c, mx_dequant(bf16_bits_to_f32((uint16_t)e2m1_to_bf16_bits((w[i >> 3] >> (4 * (i & 7))) & 0xFu)), sb, mf, false));
+        }
+      } else {
+        const uint4 a = srcp[0], bq = srcp[BB / 32];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, bq.x, bq.y, bq.z, bq.w};
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+          put_f(i, c, mx_dequant(elem_f32<KIND>((w[i >> 2] >> (8 * (i & 3))) & 0xFFu), sb, mf, KIND == TK_E5M2));
+      }
+    }
+    uint16_t* q = out + o * ostride_outer + (blk0 + b) * 32 * ostride_axis + col0 + c4;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      *reinterpret_cast<uint2*>(q + i * ostride_axis) = make_uint2(hp[i][0], hp[i][1]);
+    }
+  }
+}
+
 // ---- dispatch helpers --------------------------------------------------------------------------
 template <int SRC, int KIND>
 int32_t launch_down(const void* src, int64_t outer, int64_t L, int64_t inner, int64_t inner_last, int64_t so, int64_t sa, int64_t si,
@@ -275,6 +488,17 @@ int32_t launch_down(const void* src, int64_t outer, int64_t L, int64_t inner, in
   }
   if (si != 1 && inner != 1) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: inner stride must be 1");
   const int64_t nblk = L / 32;
+  if constexpr (sizeof(T) == 2) {
+    if (inner % 4 == 0 && sa % 4 == 0 && so % 4 == 0 && (reinterpret_cast<uintptr_t>(src) % 8) == 0 &&
+        (reinterpret_cast<uintptr_t>(out_vals) % 16) == 0) {
+      const int64_t col_tiles = cdiv(inner, kTileCols), blk_tiles = cdiv(nblk, TileGeom<KIND>::NB);
+      const int64_t grid = col_tiles * blk_tiles * outer;
+      if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_downcast: tensor too large for one launch");
+      hipLaunchKernelGGL((mx_down_tile<SRC, KIND>), dim3((unsigned)grid), dim3(kThreads), 0, st, reinterpret_cast<const uint16_t*>(s), so, sa,
+                         L, inner, inner_last, col_tiles, blk_tiles, ov, os, rounding);
+      return check_launch("mx_down_tile");
+    }
+  }
   const int64_t blk_tiles = cdiv(nblk, 4);
   const size_t esz = sizeof(T);
   const bool pair_ok = inner % 2 == 0 && sa % 2 == 0 && so % 2 == 0 && (reinterpret_cast<uintptr_t>(src) % (2 * esz)) == 0;
@@ -310,6 +534,17 @@ int32_t launch_up(const void* vals, const void* scales, int64_t outer, int64_t L
   }
   if (osi != 1 && inner != 1) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: output inner stride must be 1");
   const int64_t nblk = L / 32;
+  if constexpr (sizeof(T) == 2) {
+    if (inner % 4 == 0 && osa % 4 == 0 && oso % 4 == 0 && (reinterpret_cast<uintptr_t>(out) % 8) == 0 &&
+        (reinterpret_cast<uintptr_t>(vals) % 16) == 0) {
+      const int64_t col_tiles = cdiv(inner, kTileCols), blk_tiles = cdiv(nblk, TileGeom<KIND>::NB);
+      const int64_t grid = col_tiles * blk_tiles * outer;
+      if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_mx_upcast: tensor too large for one launch");
+      hipLaunchKernelGGL((mx_up_tile<KIND, DST>), dim3((unsigned)grid), dim3(kThreads), 0, st, v, s, L, inner, inner_last, col_tiles,
+                         blk_tiles, reinterpret_cast<uint16_t*>(o), oso, osa);
+      return check_launch("mx_up_tile");
+    }
+  }
   const int64_t blk_tiles = cdiv(nblk, 4);
   const size_t esz = sizeof(T);
   const bool pair_ok = inner % 2 == 0 && osa % 2 == 0 && oso % 2 == 0 && (reinterpret_cast<uintptr_t>(out) % (2 * esz)) == 0;
