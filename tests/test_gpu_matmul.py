@@ -235,6 +235,34 @@ def test_matmul_fp8(mods, device, m, n, k, layout, block_m, do_gather, do_scatte
     assert_allclose_gate(ref, y, what="fp8 y", max_bad_frac=1e-4 if swiglu else 0.0)
 
 
+@pytest.mark.parametrize("per_expert", [False, True])
+def test_flexpoint_input_scales(mods, device, per_expert):
+    """`FlexCtx(lhs_data=InFlexData(scale=...), rhs_data=InFlexData(scale=...))`: fp8 operands with one-element device
+    scales (per expert for the weights when the scale tensor has one entry per expert), `acc *= x_scale * w_scale`
+    before the bias (matmul_details/_matmul.py:540-547).  Oracle: dequantise with the scales, pinned GEMM oracle."""
+    mm, _, tensor = mods
+    from triton_amd.numerics import InFlexData
+    g = torch.Generator().manual_seed(31)
+    m, n, k, n_slices = 200, 256, 320, 4
+    xq = (torch.randn((m, k), generator=g) * 2).to(torch.float8_e4m3fn)
+    wq = (torch.randn((n_slices, k, n), generator=g) * 2).to(torch.float8_e4m3fn)
+    bias = torch.randn((n_slices, n), generator=g)
+    sx = torch.tensor([0.37])
+    sw = torch.tensor([0.11, 0.25, 0.5, 0.07]) if per_expert else torch.tensor([0.19])
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    flex = mm.FlexCtx(lhs_data=InFlexData(scale=sx.to(device)), rhs_data=InFlexData(scale=sw.to(device)))
+    wd = wq.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)
+    y = mm.matmul(xq.to(device), wd, bias.to(device), md, precision_config=mm.PrecisionConfig(flex_ctx=flex, out_dtype=torch.bfloat16))
+    ref = omoe.matmul(xq, wq, bias, sizes, x_row_scale=sx.expand(m), w_col_scale=sw.reshape(-1, 1).expand(n_slices, n), out_dtype=torch.bfloat16)
+    assert_close(ref, y, what="flexpoint-scaled y")
+    assert_allclose_gate(ref, y, what="flexpoint-scaled y")
+    with pytest.raises(NotImplementedError):  # output-side flexpoint needs fp8 outputs
+        from triton_amd.numerics import OutFlexData
+        mm.matmul(xq.to(device), wd, None, md, precision_config=mm.PrecisionConfig(
+            flex_ctx=mm.FlexCtx(out_data=OutFlexData(expected_scale=sx.to(device))), out_dtype=torch.bfloat16))
+
+
 @pytest.mark.parametrize("wkind", ["mxfp4", "mxfp4_tiled"])
 def test_cdna4_scale_layout_accepted(mods, device, wkind):
     """Scales pre-shuffled with the reference's `CDNA4MXScaleLayout` (what its default helper returns on this GPU,

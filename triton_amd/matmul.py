@@ -13,7 +13,8 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
 
 Options of the reference signature that this build rejects with NotImplementedError: ragged-K
 (`b_ragged_metadata`), `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
-scales, batched 3-D activations, split-k.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
+output / accumulator scales, batched 3-D activations, split-k.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
+`flex_ctx.rhs_data.scale`) are folded into the per-row / per-column scales of the epilogue.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
 MX quantiser kernel on the same stream.
 """
 from __future__ import annotations
@@ -101,9 +102,8 @@ def matmul_set_idle_sms(num_idle_sms):
     set_idle_sms(num_idle_sms)
 
 
-def _flex_is_trivial(flex: FlexCtx) -> bool:
-    return (flex.lhs_data.scale is None and flex.rhs_data.scale is None and flex.acc_data.scale is None
-            and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
+def _flex_out_is_trivial(flex: FlexCtx) -> bool:
+    return (flex.acc_data.scale is None and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
             and flex.out_data.checksum_scale is None)
 
 
@@ -194,12 +194,14 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
                               fused_activation, epilogue)
     if epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
         raise NotImplementedError(f"epilogue {epilogue.specs.name!r} is not supported (MXFP8 / MXFP4 output quantisation only)")
-    if not _flex_is_trivial(precision_config.flex_ctx):
-        raise NotImplementedError("flexpoint scales are not supported; use a/b_mx_tensor_scale for fp8 scales")
+    flex = precision_config.flex_ctx
+    if not _flex_out_is_trivial(flex):
+        raise NotImplementedError("flexpoint output / accumulator scales are not supported (outputs are bf16)")
     if precision_config.a_mx_scale is not None:
         raise NotImplementedError("MX-quantised activations (a_mx_scale) are not supported")
     if isinstance(a, Tensor):
         a = a.storage.data
+    a = flex.lhs_data.reinterpret(a)
     if a.ndim != 2:
         raise NotImplementedError("batched 3-D activations are not supported")
     nt.require_gpu(a, "a")
@@ -279,6 +281,14 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if a_ts is not None:
         a_ts = a_ts.to(torch.float32).reshape(-1).contiguous()
         assert a_ts.numel() == a.shape[0], "a_mx_tensor_scale must hold one scale per row of a"
+    if flex.lhs_data.scale is not None:
+        # flexpoint input scale (`acc *= x_scale * w_scale` before the bias, matmul_details/_matmul.py:540-547): a
+        # one-element device tensor, folded into the per-row scale the kernel already applies (no host read)
+        xs = flex.lhs_data.scale.to(torch.float32).reshape(-1)
+        if xs.numel() != 1:
+            raise NotImplementedError("per-batch flexpoint scales need batched activations, which are not supported")
+        a_ts = a_ts * xs if a_ts is not None else xs.expand(a.shape[0]).contiguous()
+    if a_ts is not None:
         d.x_row_scale = a_ts.data_ptr()
     keep = [a_ts]
     if tiled_fp8:
@@ -324,6 +334,14 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     b_ts = precision_config.b_mx_tensor_scale
     if b_ts is not None:
         b_ts = b_ts.to(torch.float32).reshape(w.shape[0], N).contiguous()
+    if flex.rhs_data.scale is not None:
+        # one scale for all experts or one per expert (PER_BATCH_W_SCALE), folded into the per-column scale
+        ws_ = flex.rhs_data.scale.to(torch.float32).reshape(-1)
+        if ws_.numel() not in (1, w.shape[0]):
+            raise ValueError(f"rhs flexpoint scale must hold 1 or {w.shape[0]} values, got {ws_.numel()}")
+        col = ws_.reshape(-1, 1).expand(w.shape[0], N)
+        b_ts = b_ts * col if b_ts is not None else col.contiguous()
+    if b_ts is not None:
         d.w_col_scale = b_ts.data_ptr()
         d.wcs_stride_e = b_ts.stride(0)
         keep.append(b_ts)
