@@ -41,19 +41,71 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__device__ inline unsigned long long wave_max_u64(unsigned long long v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    const unsigned long long o = __shfl_xor(v, off);
-    v = o > v ? o : v;
+// Wave-wide reductions with DPP lane exchanges (no LDS round trips): xor-1 and xor-2 inside a quad, mirror inside 8
+// and inside 16 lanes leave every lane with its row's result; the four rows are combined through scalar reads.
+// The result is uniform.  All 64 lanes must be active.
+#define TK_DPP_QUAD_XOR1 0xB1      /* quad_perm [1,0,3,2] */
+#define TK_DPP_QUAD_XOR2 0x4E      /* quad_perm [2,3,0,1] */
+#define TK_DPP_ROW_HALF_MIRROR 0x141
+#define TK_DPP_ROW_MIRROR 0x140
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  int x = (int)v;
+#define TK_STEP(ctrl)                                                                  \
+  {                                                                                    \
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false); \
+    x = (int)(o > (uint32_t)x ? o : (uint32_t)x);                                      \
   }
-  return v;
+  TK_STEP(TK_DPP_QUAD_XOR1)
+  TK_STEP(TK_DPP_QUAD_XOR2)
+  TK_STEP(TK_DPP_ROW_HALF_MIRROR)
+  TK_STEP(TK_DPP_ROW_MIRROR)
+#undef TK_STEP
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane(x, 0), b = (uint32_t)__builtin_amdgcn_readlane(x, 16);
+  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane(x, 32), d = (uint32_t)__builtin_amdgcn_readlane(x, 48);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
 }
 
-__device__ inline float wave_sum_f32(float v) {
+__device__ __forceinline__ float wave_sum_f32(float v) {
+  int x = __builtin_bit_cast(int, v);
+#define TK_STEP(ctrl) x = __builtin_bit_cast(int, __builtin_bit_cast(float, x) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false)));
+  TK_STEP(TK_DPP_QUAD_XOR1)
+  TK_STEP(TK_DPP_QUAD_XOR2)
+  TK_STEP(TK_DPP_ROW_HALF_MIRROR)
+  TK_STEP(TK_DPP_ROW_MIRROR)
+#undef TK_STEP
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 0)), b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 32)), d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 48));
+  return (a + b) + (c + d);
+}
+
+// Top-k of one row spread over a wave: lane l holds the order-preserving keys of experts l, l + 64, ... in hi[]
+// (0 for columns past E).  Round j picks the largest key, ties to the lowest expert index (the reference packs
+// E_pad - idx under the key for the same effect, topk_details/_topk_forward.py:27-35,61), hands it to lane j and
+// retires it.  Same selection as a stable descending sort.
+template <int EPL>
+__device__ __forceinline__ void wave_topk(uint32_t (&hi)[EPL], int k, int E, int lane, float& myval, int& myidx) {
+  uint32_t retired = 0;  // bit i: hi[i] is out of the running (columns past E from the start)
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
-  return v;
+  for (int i = 0; i < EPL; ++i) retired |= (lane + 64 * i >= E ? 1u : 0u) << i;
+  for (int j = 0; j < k; ++j) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) m = (!((retired >> i) & 1u) && hi[i] > m) ? hi[i] : m;
+    m = wave_max_u32(m);
+    int sel = -1;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const unsigned long long mask = __ballot(!((retired >> i) & 1u) && hi[i] == m);
+      if (sel < 0 && mask != 0ull) sel = 64 * i + (int)__builtin_ctzll(mask);
+    }
+    if (sel >= 0 && lane == (sel & 63)) retired |= 1u << (sel >> 6);
+    if (lane == j) {
+      myval = key_to_float(m);
+      myidx = sel;
+    }
+  }
 }
 
 template <int DT>
@@ -132,12 +184,9 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
       }
     } else {
-      unsigned long long key[EPL];
+      uint32_t key[EPL];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        const int e = lane + 64 * i;
-        key[i] = e < E ? (((unsigned long long)ordered_key(next_v[i]) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
-      }
+      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(next_v[i]) : 0u;
       if (row + 1 < row_end && row + 1 < n_rows) {
 #pragma unroll
         for (int i = 0; i < EPL; ++i) {
@@ -145,19 +194,7 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
           next_v[i] = e < E ? load_logit<DT>(p.logits, (int64_t)(row + 1) * p.stride_m + e) : 0.f;
         }
       }
-      for (int j = 0; j < k; ++j) {
-        unsigned long long best = key[0];
-#pragma unroll
-        for (int i = 1; i < EPL; ++i) best = key[i] > best ? key[i] : best;
-        best = wave_max_u64(best);
-#pragma unroll
-        for (int i = 0; i < EPL; ++i)
-          if (key[i] == best) key[i] = 0ull;
-        if (lane == j) {
-          myval = key_to_float((uint32_t)(best >> 32));
-          myidx = (int)(~(uint32_t)best);
-        }
-      }
+      wave_topk<EPL>(key, k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
@@ -169,7 +206,7 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
         for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
         vmax = m;
       } else {
-        vmax = __shfl(myval, 0);
+        vmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, myval), 0));
       }
       const float z = lane < k ? expf(myval - vmax) : 0.f;
       const float sum = wave_sum_f32(z);
@@ -433,27 +470,12 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
       }
     } else {
-      unsigned long long key[EPL];
+      uint32_t key[EPL];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        const int e = lane + 64 * i;
-        key[i] = e < E ? ((unsigned long long)ordered_key(nv[i]) << 32) | (uint32_t)(~(uint32_t)e) : 0ull;
-      }
+      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(nv[i]) : 0u;
       const int nrow = row + kScanWaves;
       if (nrow < T && nrow < n_rows) load_row(nrow);
-      for (int j = 0; j < k; ++j) {
-        unsigned long long best = key[0];
-#pragma unroll
-        for (int i = 1; i < EPL; ++i) best = key[i] > best ? key[i] : best;
-        best = wave_max_u64(best);
-#pragma unroll
-        for (int i = 0; i < EPL; ++i)
-          if (key[i] == best) key[i] = 0ull;
-        if (lane == j) {
-          myval = key_to_float((uint32_t)(best >> 32));
-          myidx = (int)(~(uint32_t)best);
-        }
-      }
+      wave_topk<EPL>(key, k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
@@ -464,7 +486,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
         for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
         vmax = m;
       } else {
-        vmax = __shfl(myval, 0);
+        vmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, myval), 0));
       }
       const float z = lane < k ? expf(myval - vmax) : 0.f;
       const float sum = wave_sum_f32(z);
