@@ -1,11 +1,13 @@
 // MX quantise / dequantise kernels for gfx950 (HBM-bound byte work).
 //
-// Two source layouts are handled without a transposed temporary:
+// Source layouts handled without a transposed temporary:
 //   rows : the quantised axis is the unit-stride one; 4 lanes share a block of 32, each holds 8
 //          consecutive elements, the block maximum is a 2-step lane exchange.
 //   cols : the quantised axis is strided and the INNER axis is unit-stride (a weight [E, K, N]
 //          quantised along K); a lane owns one or two columns and walks 32 rows, so every load of a
 //          wave is one contiguous row segment and the 32-element reduction is register-local.
+//   tile : the cols case for 16-bit tensors, with an LDS transpose so that the quantised bytes of a column move
+//          as full 128-byte lines (mx_down_tile / mx_up_tile).
 #include "mx_math.h"
 
 namespace tk {
