@@ -397,7 +397,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.y_stride_m = c.stride(0)
     d.activation = act
     d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
-    with torch.cuda.device(a.device):
+    with nt.on_device(a.device):
         nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
     del keep
     return c

@@ -125,7 +125,7 @@ def downcast_to_mxfp(x, out_dtype, axis: int, scale_dtype: torch.dtype = torch.u
             view = _collapse(src, axis)
         outer, L_, inner, so, sa, si = view
         inner_last = src.shape[-1] if axis < src.ndim - 1 else 1
-        with torch.cuda.device(src.device):
+        with nt.on_device(src.device):
             nt.check(
                 nt.lib().tk_mx_downcast(src.data_ptr(), _FLOAT_SRC[src.dtype], outer, L_, inner, inner_last, so, sa, si,
                                         y_value.storage.data.data_ptr(), y_scale.storage.data.data_ptr(),
@@ -164,7 +164,7 @@ def upcast_from_mxfp(tensor: torch.Tensor, scale: torch.Tensor, target_dtype: to
         inner = _prod(out_shape[axis + 1:])
         inner_last = out_shape[-1] if axis < ndim - 1 else 1
         kind = {torch.uint8: nt.TK_E2M1, torch.float8_e4m3fn: nt.TK_E4M3, torch.float8_e5m2: nt.TK_E5M2}[tensor.dtype]
-        with torch.cuda.device(tensor.device):
+        with nt.on_device(tensor.device):
             nt.check(
                 nt.lib().tk_mx_upcast(v.data_ptr(), s.data_ptr(), kind, outer, L, inner, inner_last, out.data_ptr(),
                                       nt.TORCH_TO_TK[target_dtype], L * inner, inner, 1, nt.stream_ptr(tensor.device)))

@@ -21,7 +21,7 @@ def quantize_fp8_rowwise(x: torch.Tensor):
     M, K = x.shape
     q = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=x.device)
     s = torch.empty((M, ), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with nt.on_device(x.device):
         nt.check(
             nt.lib().tk_quant_fp8_rows(x.data_ptr(), nt.TK_BF16, M, K, x.stride(0) if M else 0, q.data_ptr(), q.stride(0) if M else 0,
                                        s.data_ptr(), nt.stream_ptr(x.device)))

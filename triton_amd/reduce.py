@@ -71,7 +71,7 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
         scale_f = scale if scale.dtype == torch.float32 else scale.to(torch.float32)
         scale_f, ss = _bcast_strides(scale_f, x.shape)
         s_ptr = scale_f.data_ptr()
-    with torch.cuda.device(x.device):
+    with nt.on_device(x.device):
         nt.check(
             nt.lib().tk_reduce_mid(x.data_ptr(), nt.TORCH_TO_TK[x.dtype], A, K, C, x.stride(0), x.stride(1), m_ptr, *ms, s_ptr,
                                    *ss, y.data_ptr(), y.stride(0) if A else 0, nt.stream_ptr(x.device)))

@@ -52,7 +52,7 @@ def swiglu(a, alpha, precision_config, routing_data=None):
     if routing_data is not None:
         n_tokens = routing_data.expt_data.token_offs[routing_data.n_expts_tot:routing_data.n_expts_tot + 1]
     limit = precision_config.limit
-    with torch.cuda.device(a.device):
+    with nt.on_device(a.device):
         nt.check(
             nt.lib().tk_swiglu(a2.data_ptr(), nt.TORCH_TO_TK[a.dtype], M, N // 2, a2.stride(0) if M else 0, out.data_ptr(),
                                out.stride(0), float(alpha), float(limit) if limit is not None else 0.0,

@@ -55,16 +55,23 @@ def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_
         d.bitmatrix = bitmatrix_data.data_ptr()
         d.bitmatrix_stride_w = bitmatrix_data.stride(1)
     if want_meta:
-        col_sum = torch.empty((n_experts, ), dtype=torch.int32, device=dev)
-        combined = torch.empty((2 * R, ), dtype=torch.int32, device=dev)
-        ws = torch.empty((max(1, nt.lib().tk_route_workspace_bytes(T, n_experts)), ), dtype=torch.uint8, device=dev)
+        # one int32 allocation carved into the histogram, both permutations (adjacent, as the reference carves them
+        # from one [2R] buffer, bitmatrix.py:119-121), the gather index and the kernels' workspace
+        e_pad = (n_experts + 3) & ~3
+        ws_words = (max(1, nt.lib().tk_route_workspace_bytes(T, n_experts)) + 3) // 4
+        r_pad = (R + 3) & ~3
+        n_gather = r_pad if want_extras else 0
+        buf = torch.empty((e_pad + 2 * r_pad + n_gather + ws_words, ), dtype=torch.int32, device=dev)
+        col_sum = buf[:n_experts]
+        combined = buf[e_pad:e_pad + 2 * R]
+        ws = buf[e_pad + 2 * r_pad + n_gather:]
         out.update(col_sum=col_sum, col_sorted_indx=combined[:R], row_sorted_indx=combined[R:], _ws=ws)
         d.col_sum = col_sum.data_ptr()
         d.col_sorted_indx = combined.data_ptr()
         d.row_sorted_indx = combined.data_ptr() + 4 * R
         d.workspace = ws.data_ptr()
         if want_extras:
-            gather = torch.empty((R, ), dtype=torch.int32, device=dev)
+            gather = buf[e_pad + 2 * r_pad:e_pad + 2 * r_pad + R]
             d.gather_indx = gather.data_ptr()
             out["gather_indx"] = gather
             if vals is not None:
@@ -80,7 +87,7 @@ def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_
             d.block_schedule_stride = sched.stride(0) if width > 0 else 0
             d.max_n_blocks = width
     if T > 0:
-        with torch.cuda.device(dev):
+        with nt.on_device(dev):
             nt.check(nt.lib().tk_route(d, nt.stream_ptr(dev)))
     elif want_meta:
         out["col_sum"].zero_()

@@ -85,7 +85,7 @@ def make_ragged_tensor_metadata(slice_sizes, n_total_rows):
     n_slices = slice_sizes.shape[0]
     slice_sizes = slice_sizes.contiguous()
     slice_offs, block_offs, sched, width = _alloc(n_slices, n_total_rows, slice_sizes.device)
-    with torch.cuda.device(slice_sizes.device):
+    with nt.on_device(slice_sizes.device):
         nt.check(
             nt.lib().tk_ragged_metadata(nt.ptr(slice_sizes), n_slices, slice_offs.data_ptr(), block_offs.data_ptr(),
                                         block_offs.stride(0), nt.ptr(sched) if width > 0 else None,
