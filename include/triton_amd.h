@@ -161,6 +161,20 @@ int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t
                            int64_t block_offs_stride, int32_t* block_schedule, int64_t block_schedule_stride,
                            int32_t max_n_blocks, tk_stream_t stream);
 
+/*
+ * Replaces `_remap_ragged_tensor_metadata` (tk/tensor_details/ragged_tensor.py:309-381): metadata of the ragged
+ * tensor that keeps the slices with slice_map[slice] != -1, in their order.  Kept slice sizes, slice offsets and
+ * block offsets are compacted to the front (their values unchanged) and followed by -1; schedule entries of kept
+ * slices are compacted and carry slice_map[slice] as their slice id; block_offs_out[b][number of kept slices]
+ * receives the number of schedule entries kept.  Inputs and outputs have the shapes of tk_ragged_metadata's.
+ */
+int32_t tk_ragged_remap(const int32_t* slice_sizes, const int32_t* slice_offs, const int32_t* block_offs,
+                        int64_t block_offs_stride, const int32_t* block_schedule, int64_t block_schedule_stride,
+                        const int32_t* slice_map, int32_t n_slices, int32_t n_block_sizes, int32_t max_n_blocks,
+                        int32_t* slice_sizes_out, int32_t* slice_offs_out, int32_t* block_offs_out,
+                        int64_t block_offs_out_stride, int32_t* block_schedule_out, int64_t block_schedule_out_stride,
+                        tk_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Ragged expert GEMM
  * ---------------------------------------------------------------------------------------------- */

@@ -6,6 +6,8 @@ Test infrastructure only.  Follows
   * `make_ragged_tensor_metadata_torch`  .../tensor_details/ragged_tensor.py:217-253
     with `n_blocks / max_n_blocks / block_sizes` of .../ragged_tensor.py:73-89 (HIP set 16..256)
   * the routing glue of python/triton_kernels/tests/test_distributed.py:203-210
+  * `remap_ragged_tensor_metadata_torch` .../tensor_details/ragged_tensor.py:388-433 (pinned in
+    tests/test_oracle_routing.py by a hand-worked example and by rebuilding the kept slices' metadata from scratch)
 """
 from __future__ import annotations
 
@@ -114,6 +116,37 @@ def make_ragged_tensor_metadata(slice_sizes: torch.Tensor, n_total_rows: int) ->
         block_schedule_data=torch.from_numpy(np.stack(sched_rows)) if width > 0 else torch.empty(
             (len(BLOCK_SIZES), 0), dtype=torch.int32),
     )
+
+
+def remap_ragged_tensor_metadata(md: RaggedTensorMetadata, slice_map: torch.Tensor) -> RaggedTensorMetadata:
+    """ragged_tensor.py:388-433: keep the slices with `slice_map[s] != -1`, in their order.  Kept sizes, offsets and
+    block offsets move to the front unchanged, -1 behind them; schedule entries of kept slices are compacted and get
+    `slice_map[s]` as slice id; the first -1 of each block-offset row is replaced by the number of entries kept."""
+    smap = slice_map.detach().to("cpu").to(torch.int64).numpy()
+    n = smap.shape[0]
+    keep = smap != -1
+
+    def compact(vals, mask):
+        vals = np.asarray(vals, dtype=np.int64)
+        return np.concatenate([vals[mask], np.full(int((~mask).sum()), -1, dtype=np.int64)])
+
+    sizes = compact(md.slice_sizes.numpy(), keep)
+    keep1 = np.concatenate([keep, [False]])
+    offs = compact(md.slice_offs.numpy(), keep1)
+    bo_rows, bs_rows = [], []
+    for i in range(md.block_offs_data.shape[0]):
+        bo = compact(md.block_offs_data[i].numpy(), keep1)
+        sched = md.block_schedule_data[i].numpy().astype(np.int64)
+        valid = sched != -1
+        slice_id = np.where(valid, sched & 0xFFFF, 0)
+        kept = valid & keep[slice_id]
+        new = (sched & 0xFFFF0000) | np.where(kept, smap[slice_id], 0)
+        out = compact(new, kept)
+        bo[int(np.nonzero(bo == -1)[0][0])] = int(kept.sum())
+        bo_rows.append(bo.astype(np.int32))
+        bs_rows.append(out.astype(np.int32))
+    return RaggedTensorMetadata(torch.from_numpy(sizes.astype(np.int32)), torch.from_numpy(offs.astype(np.int32)),
+                                torch.from_numpy(np.stack(bo_rows)), torch.from_numpy(np.stack(bs_rows)))
 
 
 @dataclass

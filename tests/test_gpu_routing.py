@@ -165,3 +165,50 @@ def test_baseline_router_shape(tk, device):
         assert_equal(r.meta.col_sorted_indx, sm.mask_metadata.col_sorted_indx, "col_sorted")
         assert_equal(r.meta.row_sorted_indx, sm.mask_metadata.row_sorted_indx, "row_sorted")
         assert_close(r.vals, sm.vals, what="vals")
+
+
+@pytest.mark.parametrize("n_slices", [9, 32, 911, 1025])
+def test_remap_ragged_tensor_metadata(device, n_slices):
+    """Mirrors tests/test_tensor.py:259-277 of the reference: random sizes with an empty slice, a random permutation as
+    slice map with five entries dropped; every output tensor equals the oracle's."""
+    from oracle import routing as ort
+    from triton_amd.tensor import make_ragged_tensor_metadata, remap_ragged_tensor_metadata
+    g = torch.Generator().manual_seed(n_slices)
+    max_slice_size = 200
+    n_total_rows = max_slice_size * n_slices
+    sizes = torch.randint(0, max_slice_size, (n_slices, ), dtype=torch.int32, generator=g)
+    sizes[int(torch.randint(0, n_slices, (1, ), generator=g))] = 0
+    smap = torch.randperm(n_slices, generator=g).to(torch.int32)
+    smap[torch.randint(0, n_slices, (5, ), generator=g)] = -1
+    md = make_ragged_tensor_metadata(sizes.to(device), n_total_rows)
+    got = remap_ragged_tensor_metadata(md, smap.to(device))
+    ref = ort.remap_ragged_tensor_metadata(ort.make_ragged_tensor_metadata(sizes, n_total_rows), smap)
+    assert torch.equal(got.slice_sizes.cpu(), ref.slice_sizes)
+    assert torch.equal(got.slice_offs.cpu(), ref.slice_offs)
+    assert torch.equal(got.block_offs_data.cpu(), ref.block_offs_data)
+    assert torch.equal(got.block_schedule_data.cpu(), ref.block_schedule_data)
+
+
+def test_matmul_on_remapped_metadata(device):
+    """The expert-parallel use (tests/test_distributed.py:236-241 of the reference): global metadata restricted to a
+    rank's experts, the rank's weights only; rows of the kept experts sit at their global positions."""
+    from oracle import moe as omoe
+    from oracle.checks import assert_close
+    from triton_amd.matmul import matmul
+    from triton_amd.tensor import make_ragged_tensor_metadata, remap_ragged_tensor_metadata
+    g = torch.Generator().manual_seed(5)
+    E, K, N = 8, 256, 192
+    sizes = torch.tensor([40, 17, 0, 130, 33, 5, 64, 11], dtype=torch.int32)
+    M = int(sizes.sum())
+    local = [1, 3, 4, 6]
+    smap = torch.full((E, ), -1, dtype=torch.int32)
+    smap[local] = torch.arange(len(local), dtype=torch.int32)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    w = (torch.randn((E, K, N), generator=g) * 0.1).to(torch.bfloat16)
+    md = remap_ragged_tensor_metadata(make_ragged_tensor_metadata(sizes.to(device), M), smap.to(device))
+    y = matmul(x.to(device), w[local].to(device), None, md).cpu()
+    offs = torch.cumsum(torch.cat([torch.zeros(1, dtype=torch.int64), sizes.long()]), 0)
+    for e in local:
+        lo, hi = int(offs[e]), int(offs[e + 1])
+        ref = omoe.matmul(x[lo:hi], w[e:e + 1], None, torch.tensor([hi - lo]))
+        assert_close(ref, y[lo:hi], what=f"rows of expert {e}")

@@ -137,3 +137,31 @@ def test_routing_glue():
     assert torch.equal(r.scatter_indx.long(), cs)
     assert torch.equal(r.gammas, r.vals.reshape(-1)[cs])
     assert torch.allclose(r.vals.sum(-1), torch.ones(T), atol=1e-6)
+
+
+def test_remap_ragged_metadata_hand_example_and_rebuild():
+    """`remap_ragged_tensor_metadata` (ragged_tensor.py:388-433).  Hand-worked: sizes [15, 17, 0, 127] keeping slices 1 and 3
+    as local 0 and 1.  Block size 16: blocks per slice [1, 2, 0, 8], offsets [0, 1, 3, 3, 11]; kept offsets are those of
+    slices 1 and 3 (1 and 3), then the 10 entries kept, then -1.  Independent check: the compacted schedule equals the
+    schedule built from scratch for the kept sizes [17, 127], entry for entry."""
+    from oracle import routing as ort
+    sizes = torch.tensor([15, 17, 0, 127], dtype=torch.int32)
+    md = ort.make_ragged_tensor_metadata(sizes, 159)
+    smap = torch.tensor([-1, 0, -1, 1], dtype=torch.int32)
+    r = ort.remap_ragged_tensor_metadata(md, smap)
+    assert r.slice_sizes.tolist() == [17, 127, -1, -1]
+    assert r.slice_offs.tolist() == [15, 32, -1, -1, -1]
+    assert r.block_offs_data[0].tolist() == [1, 3, 10, -1, -1]  # block size 16
+    assert r.block_offs_data[3].tolist() == [1, 2, 2, -1, -1]  # block size 128: one block each
+    s16 = r.block_schedule_data[0].tolist()
+    assert s16[:10] == [(0 << 16) | 0, (1 << 16) | 0] + [(b << 16) | 1 for b in range(8)] and set(s16[10:]) <= {-1}
+    fresh = ort.make_ragged_tensor_metadata(torch.tensor([17, 127], dtype=torch.int32), 159)
+    for i in range(len(ort.BLOCK_SIZES)):
+        n = int(fresh.block_offs_data[i][-1])
+        assert r.block_schedule_data[i][:n].tolist() == fresh.block_schedule_data[i][:n].tolist()
+        assert int(r.block_offs_data[i][2]) == n
+    # a permuting map only renames the slice ids inside the schedule
+    smap2 = torch.tensor([2, -1, 0, 1], dtype=torch.int32)
+    r2 = ort.remap_ragged_tensor_metadata(md, smap2)
+    assert r2.slice_sizes.tolist() == [15, 0, 127, -1]
+    assert [e & 0xFFFF for e in r2.block_schedule_data[3].tolist() if e != -1] == [2, 1]

@@ -414,6 +414,81 @@ __global__ __launch_bounds__(kScanThreads) void ragged_metadata_kernel(const int
   ragged_metadata(slice_sizes, E, nullptr, r, true);
 }
 
+// ---- remapping ragged metadata to a subset of the slices ------------------------------------------------
+// Order-preserving compaction by a 1024-thread workgroup: out[rank(i)] = value(i) for the kept i, -1 behind them.
+// `f(i, v)` yields element i's value and whether it is kept.  Returns the number kept (uniform).
+template <class F>
+__device__ __forceinline__ int compact_block(int32_t* out, int n, int* wave_tot, F&& f) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int base = 0;
+  for (int start = 0; start < n; start += kScanThreads) {
+    const int i = start + threadIdx.x;
+    int32_t v = -1;
+    const bool keep = i < n && f(i, v);
+    const unsigned long long mask = __ballot(keep);
+    if (lane == 0) wave_tot[wave] = __builtin_popcountll(mask);
+    __syncthreads();
+    int before = 0, total = 0;
+    for (int w = 0; w < kScanThreads / 64; ++w) {
+      const int t = wave_tot[w];
+      before += w < wave ? t : 0;
+      total += t;
+    }
+    if (keep) out[base + before + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = v;
+    base += total;
+    __syncthreads();
+  }
+  for (int i = base + threadIdx.x; i < n; i += kScanThreads) out[i] = -1;
+  return base;
+}
+
+struct RemapParams {
+  const int32_t* slice_sizes;
+  const int32_t* slice_offs;
+  const int32_t* block_offs;
+  int64_t block_offs_stride;
+  const int32_t* block_sched;
+  int64_t block_sched_stride;
+  const int32_t* slice_map;
+  int32_t n_slices, max_n_blocks;
+  int32_t* slice_sizes_out;
+  int32_t* slice_offs_out;
+  int32_t* block_offs_out;
+  int64_t block_offs_out_stride;
+  int32_t* block_sched_out;
+  int64_t block_sched_out_stride;
+};
+
+// Workgroup 0 compacts the slice sizes and offsets; workgroup 1 + b the block offsets and the block schedule of
+// block size b, whose entries get the slice's new id; the count of the schedule entries kept goes behind the kept
+// block offsets (tensor_details/ragged_tensor.py:309-345 of the reference).
+__global__ __launch_bounds__(kScanThreads) void ragged_remap_kernel(const RemapParams p) {
+  __shared__ int wave_tot[kScanThreads / 64];
+  const int n = p.n_slices;
+  const int32_t* map = p.slice_map;
+  auto kept_slice = [&](int i) { return i < n && map[i] != -1; };
+  if (blockIdx.x == 0) {
+    compact_block(p.slice_sizes_out, n, wave_tot, [&](int i, int32_t& v) { v = p.slice_sizes[i]; return kept_slice(i); });
+    compact_block(p.slice_offs_out, n + 1, wave_tot, [&](int i, int32_t& v) { v = p.slice_offs[i]; return kept_slice(i); });
+    return;
+  }
+  const int b = blockIdx.x - 1;
+  const int32_t* bo = p.block_offs + b * p.block_offs_stride;
+  const int32_t* bs = p.block_sched + b * p.block_sched_stride;
+  int32_t* bo_out = p.block_offs_out + b * p.block_offs_out_stride;
+  const int n_kept = compact_block(bo_out, n + 1, wave_tot, [&](int i, int32_t& v) { v = bo[i]; return kept_slice(i); });
+  const int n_blocks = compact_block(p.block_sched_out + b * p.block_sched_out_stride, p.max_n_blocks, wave_tot, [&](int i, int32_t& v) {
+    const uint32_t e = (uint32_t)bs[i];
+    const uint32_t slice = e & 0xFFFFu;
+    if (slice == 0xFFFFu || (int)slice >= n) return false;  // unused tail of the schedule
+    const int32_t to = map[slice];
+    v = (int32_t)((e & 0xFFFF0000u) | ((uint32_t)to & 0xFFFFu));
+    return to != -1;
+  });
+  __syncthreads();
+  if (threadIdx.x == 0) bo_out[n_kept] = n_blocks;
+}
+
 // ---- whole routing pass in ONE workgroup (small batches) ------------------------------------------
 // For T*k <= kSmallEntries the three phases run back to back in a single 1024-thread workgroup: the waves take
 // rows round-robin for the top-k, the selected expert ids stay in LDS, the histogram is built with LDS atomics,
@@ -802,4 +877,35 @@ extern "C" int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slic
   ro.max_n_blocks = max_n_blocks;
   hipLaunchKernelGGL(ragged_metadata_kernel, dim3(1), dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), slice_sizes, n_slices, ro);
   return check_launch("ragged_metadata_kernel");
+}
+
+extern "C" int32_t tk_ragged_remap(const int32_t* slice_sizes, const int32_t* slice_offs, const int32_t* block_offs,
+                                   int64_t block_offs_stride, const int32_t* block_schedule, int64_t block_schedule_stride,
+                                   const int32_t* slice_map, int32_t n_slices, int32_t n_block_sizes, int32_t max_n_blocks,
+                                   int32_t* slice_sizes_out, int32_t* slice_offs_out, int32_t* block_offs_out,
+                                   int64_t block_offs_out_stride, int32_t* block_schedule_out, int64_t block_schedule_out_stride,
+                                   tk_stream_t stream) {
+  if (n_slices < 0 || n_block_sizes < 0 || max_n_blocks < 0) return fail(TK_ERR_INVALID, "tk_ragged_remap: negative size");
+  if (n_slices >= 65536) return fail(TK_ERR_INVALID, "tk_ragged_remap: at most 65535 slices");
+  if (!slice_offs || !slice_offs_out || (n_slices > 0 && (!slice_sizes || !slice_map || !slice_sizes_out)) ||
+      (n_block_sizes > 0 && (!block_offs || !block_offs_out)) || (n_block_sizes > 0 && max_n_blocks > 0 && (!block_schedule || !block_schedule_out)))
+    return fail(TK_ERR_INVALID, "tk_ragged_remap: null pointer");
+  RemapParams p;
+  p.slice_sizes = slice_sizes;
+  p.slice_offs = slice_offs;
+  p.block_offs = block_offs;
+  p.block_offs_stride = block_offs_stride;
+  p.block_sched = block_schedule;
+  p.block_sched_stride = block_schedule_stride;
+  p.slice_map = slice_map;
+  p.n_slices = n_slices;
+  p.max_n_blocks = max_n_blocks;
+  p.slice_sizes_out = slice_sizes_out;
+  p.slice_offs_out = slice_offs_out;
+  p.block_offs_out = block_offs_out;
+  p.block_offs_out_stride = block_offs_out_stride;
+  p.block_sched_out = block_schedule_out;
+  p.block_sched_out_stride = block_schedule_out_stride;
+  hipLaunchKernelGGL(ragged_remap_kernel, dim3(1 + n_block_sizes), dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), p);
+  return check_launch("ragged_remap_kernel");
 }

@@ -161,6 +161,20 @@ def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, pre
     return vals
 
 
+def _localise_remapped_metadata(md: RaggedTensorMetadata, n_local: int, n_rows: int) -> RaggedTensorMetadata:
+    """Metadata from `remap_ragged_tensor_metadata` as the kernels need it.  The reference's kernel takes the weight
+    tensor's slice count as the number of slices (`n_valid_slices`, matmul.py:658), looks rows up through the kept
+    slices' unchanged offsets and never uses the (source-tensor) block offsets for scheduling; the kernels here order
+    tiles by them, so block offsets and schedule are rebuilt for the `n_local` kept slices (one small launch) while
+    sizes and row offsets are taken as remapped.  As in the reference this assumes that `slice_map` numbers the kept
+    slices 0..n_local-1 in their original order."""
+    from .tensor_details.ragged_tensor import make_ragged_tensor_metadata
+    assert n_local <= md.n_slices, f"{n_local} weight slices for metadata remapped from {md.n_slices} slices"
+    sizes = md.slice_sizes[:n_local].clamp_min(0)
+    local = make_ragged_tensor_metadata(sizes, n_rows)
+    return RaggedTensorMetadata(sizes, md.slice_offs[:n_local + 1], local.block_offs_data, local.block_schedule_data)
+
+
 def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
            b_ragged_metadata: RaggedTensorMetadata | None = None, gather_indx: torch.Tensor | None = None,
            scatter_indx: torch.Tensor | None = None, precision_config: PrecisionConfig | None = None,
@@ -240,6 +254,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     K = a.shape[-1]
     assert K == K_W, f"reduction dims differ: a has K={K}, b has K={K_W}"
     is_ragged = a_ragged_metadata is not None
+    if is_ragged and getattr(a_ragged_metadata, "remapped_from", None) is not None:
+        a_ragged_metadata = _localise_remapped_metadata(a_ragged_metadata, w.shape[0], M)
     n_slices = a_ragged_metadata.n_slices if is_ragged else w.shape[0]
     if not is_ragged and w.shape[0] != 1:
         raise NotImplementedError("batched weights need ragged metadata")

@@ -2,8 +2,8 @@
 
 A ragged tensor is a stack of 2-D slices (one per expert) sharing the column count.  The metadata
 holds, for every row-block size a GEMM may use (16..256), where each slice's blocks start and the
-flat schedule of (block, slice) pairs.  `remap_ragged_tensor_metadata` (expert-parallel only) is not
-part of this build.
+flat schedule of (block, slice) pairs.  `remap_ragged_tensor_metadata` restricts the metadata to a subset
+of the slices (the local experts of an expert-parallel rank).
 """
 from __future__ import annotations
 
@@ -93,5 +93,30 @@ def make_ragged_tensor_metadata(slice_sizes, n_total_rows):
     return RaggedTensorMetadata(slice_sizes, slice_offs, block_offs, sched)
 
 
-def remap_ragged_tensor_metadata(*args, **kwargs):
-    raise NotImplementedError("remap_ragged_tensor_metadata is expert-parallel (multi-GPU) only and is not part of this build")
+def remap_ragged_tensor_metadata(src_ragged_tensor_metadata: RaggedTensorMetadata, slice_map: torch.Tensor) -> RaggedTensorMetadata:
+    """Metadata of the ragged tensor made of the slices with `slice_map[slice_id] != -1` (ragged_tensor.py:348-381 of the
+    reference; the expert-parallel step uses it to keep a rank's own experts).  Kept sizes / offsets keep their values
+    and move to the front, schedule entries get `slice_map[slice_id]` as their slice id."""
+    md = src_ragged_tensor_metadata
+    assert slice_map.ndim == 1
+    assert slice_map.shape[0] == md.slice_sizes.shape[0]
+    assert slice_map.dtype == torch.int32
+    nt.require_gpu(slice_map, "slice_map")
+    n_slices = md.slice_sizes.shape[0]
+    dev = md.slice_sizes.device
+    n_bs, width = md.block_offs_data.shape[0], md.block_schedule_data.shape[-1]
+    slice_sizes = torch.empty((n_slices, ), dtype=torch.int32, device=dev)
+    offs = torch.empty((n_bs + 1, n_slices + 1), dtype=torch.int32, device=dev)
+    sched = torch.empty((n_bs, width), dtype=torch.int32, device=dev)
+    src_sizes, src_offs, smap = md.slice_sizes.contiguous(), md.slice_offs.contiguous(), slice_map.contiguous()
+    bo, bs = md.block_offs_data, md.block_schedule_data
+    assert bo.stride(-1) == 1 and (width == 0 or bs.stride(-1) == 1)
+    with nt.on_device(dev):
+        nt.check(
+            nt.lib().tk_ragged_remap(nt.ptr(src_sizes), nt.ptr(src_offs), nt.ptr(bo), bo.stride(0), nt.ptr(bs) if width > 0 else None,
+                                     bs.stride(0) if width > 0 else 0, nt.ptr(smap), n_slices, n_bs, width, nt.ptr(slice_sizes),
+                                     offs[0].data_ptr(), offs[1:].data_ptr(), offs.stride(0), nt.ptr(sched) if width > 0 else None,
+                                     sched.stride(0) if width > 0 else 0, nt.stream_ptr(dev)))
+    out = RaggedTensorMetadata(slice_sizes, offs[0], offs[1:], sched)
+    out.remapped_from = n_slices  # tells `matmul` that block offsets are those of the source tensor, not a running sum
+    return out
