@@ -19,6 +19,7 @@
 //     and is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 right before the MFMA;
 //   * the rows of a tile are dealt to the WM row-waves in interleaved 16-row fragments and fragments
 //     past the expert's last row are skipped, so a nearly empty row block costs almost no MFMA time.
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -1335,6 +1336,19 @@ int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
 }
 
 // compute units of the current device (cached per device id)
+// Raises a kernel's dynamic LDS limit above 64 KiB, once per device (bit d of `done` = done on device d).  Threads
+// racing through the first call set the same value twice, which is harmless.
+inline int32_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
+  if (bytes <= 64 * 1024) return TK_OK;
+  int dev = 0;
+  const bool known = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64;
+  if (known && (done.load(std::memory_order_acquire) >> dev & 1ull)) return TK_OK;
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
+  if (known) done.fetch_or(1ull << dev, std::memory_order_release);
+  return TK_OK;
+}
+
 inline int device_cu_count() {
   static int cached[64] = {0};
   int dev = 0;
@@ -1361,12 +1375,8 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   const int64_t resident = (int64_t)device_cu_count() * per_cu;
   if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
-    static bool attr_done = false;
-    if (!attr_done && LDS_BYTES > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
-      attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256 * G), LDS_BYTES, st, q);
     return check_launch("moe_gemm_mxn_kernel");
   };
@@ -1387,12 +1397,8 @@ int32_t launch_f8n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   const int64_t resident = (int64_t)device_cu_count();
   if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
-    static bool attr_done = false;
-    if (!attr_done && LDS_BYTES > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
-      attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
     return check_launch("moe_gemm_f8n_kernel");
   };
@@ -1413,12 +1419,8 @@ int32_t launch_cfg(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   auto launch = [&](auto kern) -> int32_t {
-    static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
-    if (!attr_done && LDS_BYTES > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-      if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", LDS_BYTES, hipGetErrorString(e));
-      attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), LDS_BYTES, st, q);
     return check_launch("moe_gemm_kernel");
   };
