@@ -251,3 +251,48 @@ def test_layer_graph_replays_match_eager(api, device, T):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {i} differs from the eager result"
+
+
+def test_config5_full_shape_properties(api, device):
+    """Full Mixtral-shaped FP8 layer (8192 tokens, top-2 of 8 experts, W1 [8, 4096, 28672], W2 [8, 14336, 4096] e4m3 in the
+    tiled layout, per-channel weight scales, per-token activation scales).  The oracle is too slow for the whole layer,
+    so: (1) routing bit-exact against the oracle, (2) the first GEMM + swiglu against the oracle on the first 48 rows of
+    two experts, (3) permuting the tokens permutes the output rows exactly."""
+    from oracle import routing as ort
+    from triton_kernels.tensor import convert_layout, wrap_torch_tensor
+    from triton_kernels.tensor_details.layout import make_default_matmul_fp8_w_layout
+    T, d, E, k, f2 = 8192, 4096, 8, 2, 28672
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g)
+    dev = device
+    torch.manual_seed(4)
+
+    def qw(kdim, ndim):  # e4m3 weights [E, K, N] with stride 1 along K, per-column scales [E, N]; built on the device
+        q = torch.empty((E, ndim, kdim), dtype=torch.float8_e4m3fn, device=dev)
+        s = torch.empty((E, ndim), dtype=torch.float32, device=dev)
+        for e in range(E):
+            w = torch.randn((ndim, kdim), device=dev) * 0.02
+            s[e] = w.abs().amax(dim=1) / 448.0
+            q[e] = (w / s[e][:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
+        return q.transpose(1, 2), s
+
+    w1, s1 = qw(d, f2)
+    w2, s2 = qw(f2 // 2, d)
+    w1t = convert_layout(wrap_torch_tensor(w1), make_default_matmul_fp8_w_layout())
+    w2t = convert_layout(wrap_torch_tensor(w2), make_default_matmul_fp8_w_layout())
+    pc = lambda s: api.PrecisionConfig(b_mx_tensor_scale=s, out_dtype=torch.bfloat16)
+    out, rdata, h = _layer(api, dev, x, logits, k, w1t, None, w2t, None, pc(s1), pc(s2), fp8=True)
+    rr = ort.routing(logits, k)
+    assert_equal(rr.indx, rdata.expt_indx.to(torch.int32), "indx")
+    assert_equal(rr.meta.col_sum, rdata.expt_hist, "histogram")
+    xq, sx = omoe.quantize_fp8_rowwise(x)
+    for e in (0, E - 1):
+        lo = int(rr.ragged.slice_offs[e])
+        tok = rr.gather_indx[lo:lo + 48].long()
+        he = omoe.matmul(xq[tok], w1[e:e + 1].cpu(), None, torch.tensor([48]), x_row_scale=sx[tok], w_col_scale=s1[e:e + 1].cpu(),
+                         out_dtype=torch.float32)
+        assert_close(omoe.swiglu(he, 1.702, 7.0).to(torch.bfloat16), h[lo:lo + 48], maxtol=3e-2, what=f"expert {e} hidden")
+    perm = torch.randperm(T, generator=g)
+    out_p, _, _ = _layer(api, dev, x[perm], logits[perm], k, w1t, None, w2t, None, pc(s1), pc(s2), fp8=True)
+    assert torch.equal(out_p.cpu(), out.cpu()[perm]), "token permutation must permute the output rows exactly"
