@@ -152,6 +152,15 @@ int64_t tk_route_workspace_bytes(int32_t n_tokens, int32_t n_experts);
 int32_t tk_route(const tk_route_desc* desc, tk_stream_t stream);
 
 /*
+ * Replaces `_topk_backward` (tk/topk_details/_topk_backward.py:5-51, launched by tk/topk.py:76-85): gradient of the
+ * kept logits' softmax (or of the plain selection) scattered back into dx [n_tokens, n_experts]; every other element
+ * of dx, and every row >= n_rows, is zero.  x, dy, dx share `dtype` (fp32 / bf16 / fp16); strides in elements.
+ */
+int32_t tk_topk_backward(const void* x, int32_t dtype, int64_t stride_xm, const int16_t* indx, int64_t stride_im, const void* dy,
+                         int64_t stride_dym, void* dx, int64_t stride_dxm, int32_t n_tokens, int32_t n_experts, int32_t k,
+                         int32_t apply_softmax, int32_t n_rows, const int32_t* n_rows_ptr, tk_stream_t stream);
+
+/*
  * Replaces `_ragged_tensor_metadata_memset` + `_ragged_tensor_metadata_compute`
  * (tk/tensor_details/ragged_tensor.py:183-210): slice_offs = [0] + cumsum(slice_sizes); for block sizes
  * 16..256: block_offs = [0] + cumsum(ceil(slice_sizes / bs)) and block_schedule[offs[s] + b] =

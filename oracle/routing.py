@@ -6,6 +6,8 @@ Test infrastructure only.  Follows
   * `make_ragged_tensor_metadata_torch`  .../tensor_details/ragged_tensor.py:217-253
     with `n_blocks / max_n_blocks / block_sizes` of .../ragged_tensor.py:73-89 (HIP set 16..256)
   * the routing glue of python/triton_kernels/tests/test_distributed.py:203-210
+  * `_topk_backward`                     .../topk_details/_topk_backward.py:5-51 (pinned against torch autograd of the
+    forward oracle in tests/test_oracle_routing.py)
   * `remap_ragged_tensor_metadata_torch` .../tensor_details/ragged_tensor.py:388-433 (pinned in
     tests/test_oracle_routing.py by a hand-worked example and by rebuilding the kept slices' metadata from scratch)
 """
@@ -116,6 +118,27 @@ def make_ragged_tensor_metadata(slice_sizes: torch.Tensor, n_total_rows: int) ->
         block_schedule_data=torch.from_numpy(np.stack(sched_rows)) if width > 0 else torch.empty(
             (len(BLOCK_SIZES), 0), dtype=torch.int32),
     )
+
+
+def topk_backward(x: torch.Tensor, indx: torch.Tensor, dy_vals: torch.Tensor, apply_softmax: bool = True,
+                  n_rows: int | None = None) -> torch.Tensor:
+    """_topk_backward.py:5-51: dx is zero except at the kept columns, where it is `y * (dy - sum(y * dy))` with
+    `y = softmax(x[kept])` in fp32 (or `dy` without softmax); result in x's dtype.  Rows >= n_rows stay zero."""
+    xf = x.detach().to("cpu").to(torch.float32)
+    dy = dy_vals.detach().to("cpu").to(torch.float32)
+    ix = indx.detach().to("cpu").to(torch.int64)
+    T = xf.shape[0]
+    rows = T if n_rows is None else int(n_rows)
+    dx = torch.zeros_like(xf)
+    if rows > 0:
+        kept = torch.gather(xf[:rows], 1, ix[:rows])
+        if apply_softmax:
+            y = torch.softmax(kept, dim=1)
+            g = y * (dy[:rows] - (y * dy[:rows]).sum(dim=1, keepdim=True))
+        else:
+            g = dy[:rows]
+        dx[:rows].scatter_(1, ix[:rows], g)
+    return dx.to(x.dtype)
 
 
 def remap_ragged_tensor_metadata(md: RaggedTensorMetadata, slice_map: torch.Tensor) -> RaggedTensorMetadata:

@@ -212,3 +212,29 @@ def test_matmul_on_remapped_metadata(device):
         lo, hi = int(offs[e]), int(offs[e + 1])
         ref = omoe.matmul(x[lo:hi], w[e:e + 1], None, torch.tensor([hi - lo]))
         assert_close(ref, y[lo:hi], what=f"rows of expert {e}")
+
+
+@pytest.mark.parametrize("T, E, k", [(1, 8, 2), (300, 200, 8), (4096, 128, 4), (77, 1000, 32)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("apply_softmax", [True, False])
+def test_topk_backward(device, T, E, k, dt, apply_softmax):
+    """`topk_backward` (topk.py:76-85, _topk_backward.py:5-51) against the oracle, and through autograd of `topk`."""
+    from triton_amd.topk import topk, topk_backward
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn((T, E), generator=g).to(dt)
+    dy = torch.randn((T, k), generator=g).to(dt)
+    _, indx, _ = ort.topk(x, k, apply_softmax)
+    n_rows = None if T < 100 else T - 5
+    dx = topk_backward(x.to(device), indx.to(torch.int16).to(device), dy.to(device), k, n_rows, apply_softmax)
+    ref = ort.topk_backward(x, indx, dy, apply_softmax, n_rows)
+    assert dx.dtype == dt and dx.shape == x.shape
+    assert torch.equal((dx.cpu() != 0), (ref != 0)) or dt == torch.bfloat16  # same support (bf16 may round tiny values to 0)
+    tol = dict(rtol=2e-5, atol=1e-6) if dt == torch.float32 else dict(rtol=2e-2, atol=1e-3)
+    assert torch.allclose(dx.cpu().float(), ref.float(), **tol)
+    # through autograd: d/dx of sum(vals * dy)
+    xg = x.to(device).requires_grad_()
+    sm = topk(xg, k, apply_softmax=apply_softmax)
+    assert_equal(indx, sm.indx.to(torch.int32), "indx")
+    (sm.vals.float() * dy.to(device).float()).sum().backward()
+    full = ort.topk_backward(x, indx, dy, apply_softmax)
+    assert torch.allclose(xg.grad.cpu().float(), full.float(), **tol)

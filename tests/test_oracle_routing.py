@@ -165,3 +165,23 @@ def test_remap_ragged_metadata_hand_example_and_rebuild():
     r2 = ort.remap_ragged_tensor_metadata(md, smap2)
     assert r2.slice_sizes.tolist() == [15, 0, 127, -1]
     assert [e & 0xFFFF for e in r2.block_schedule_data[3].tolist() if e != -1] == [2, 1]
+
+
+@pytest.mark.parametrize("apply_softmax", [True, False])
+def test_topk_backward_matches_autograd(apply_softmax):
+    """The backward oracle against torch autograd of the forward oracle's definition (values = softmax over the kept
+    logits, topk.py:160-174): an independent derivation of the same gradient."""
+    from oracle import routing as ort
+    g = torch.Generator().manual_seed(3)
+    T, E, k = 37, 50, 4
+    x = torch.randn((T, E), generator=g, dtype=torch.float64).requires_grad_()
+    _, indx, _ = ort.topk(x.detach().float(), k, apply_softmax)
+    dy = torch.randn((T, k), generator=g, dtype=torch.float64)
+    kept = torch.gather(x, 1, indx.long())
+    vals = torch.softmax(kept, dim=1) if apply_softmax else kept
+    (vals * dy).sum().backward()
+    got = ort.topk_backward(x.detach().float(), indx, dy.float(), apply_softmax)
+    assert torch.allclose(got.double(), x.grad, rtol=1e-5, atol=1e-6)
+    assert int((got != 0).sum(dim=1).max()) <= k
+    part = ort.topk_backward(x.detach().float(), indx, dy.float(), apply_softmax, n_rows=10)
+    assert torch.equal(part[:10], got[:10]) and not part[10:].any()

@@ -414,6 +414,54 @@ __global__ __launch_bounds__(kScanThreads) void ragged_metadata_kernel(const int
   ragged_metadata(slice_sizes, E, nullptr, r, true);
 }
 
+// ---- top-k backward ---------------------------------------------------------------------------------------
+// dx[row, :] = 0 except dx[row, indx[row, j]] = y_j * (dy_j - sum_i y_i dy_i) with y = softmax of the k kept logits
+// (recomputed in fp32), or dy_j without softmax (topk_details/_topk_backward.py:5-51 of the reference).  One wave per
+// row; every dx element is written once, by the lane that owns its column.
+template <int DT>
+__global__ __launch_bounds__(256) void topk_backward_kernel(const void* x, int64_t stride_xm, const int16_t* indx, int64_t stride_im,
+                                                            const void* dy, int64_t stride_dym, void* dx, int64_t stride_dxm, int T,
+                                                            int E, int k, int apply_softmax, int n_rows_imm, const int32_t* n_rows_ptr) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  const int n_rows = n_rows_ptr ? *n_rows_ptr : n_rows_imm;
+  int idx = -1;
+  float g = 0.f;
+  if (row < n_rows) {
+    float xv = -INFINITY, dyv = 0.f;
+    if (lane < k) {
+      idx = indx[(int64_t)row * stride_im + lane];
+      if (idx < 0 || idx >= E) idx = -1;
+      if (idx >= 0) {
+        xv = load_logit<DT>(x, (int64_t)row * stride_xm + idx);
+        dyv = load_logit<DT>(dy, (int64_t)row * stride_dym + lane);
+      }
+    }
+    g = dyv;
+    if (apply_softmax) {
+      float m = xv;
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+      const float z = idx >= 0 ? expf(xv - m) : 0.f;
+      const float sum = wave_sum_f32(z);
+      const float y = sum > 0.f ? z / sum : 0.f;
+      const float s = wave_sum_f32(y * dyv);
+      g = y * (dyv - s);
+    }
+  }
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    float out = 0.f;
+    for (int j = 0; j < k; ++j) {
+      const int ij = __shfl(idx, j);
+      const float gj = __shfl(g, j);
+      out = (ij == e) ? gj : out;
+    }
+    if (e < E) store_val<DT>(dx, (int64_t)row * stride_dxm + e, out);
+  }
+}
+
 // ---- remapping ragged metadata to a subset of the slices ------------------------------------------------
 // Order-preserving compaction by a 1024-thread workgroup: out[rank(i)] = value(i) for the kept i, -1 behind them.
 // `f(i, v)` yields element i's value and whether it is kept.  Returns the number kept (uniform).
@@ -908,4 +956,26 @@ extern "C" int32_t tk_ragged_remap(const int32_t* slice_sizes, const int32_t* sl
   p.block_sched_out_stride = block_schedule_out_stride;
   hipLaunchKernelGGL(ragged_remap_kernel, dim3(1 + n_block_sizes), dim3(kScanThreads), 0, static_cast<hipStream_t>(stream), p);
   return check_launch("ragged_remap_kernel");
+}
+
+extern "C" int32_t tk_topk_backward(const void* x, int32_t dtype, int64_t stride_xm, const int16_t* indx, int64_t stride_im, const void* dy,
+                                    int64_t stride_dym, void* dx, int64_t stride_dxm, int32_t n_tokens, int32_t n_experts, int32_t k,
+                                    int32_t apply_softmax, int32_t n_rows, const int32_t* n_rows_ptr, tk_stream_t stream) {
+  if (n_tokens < 0 || n_experts <= 0 || k <= 0 || k > 64) return fail(TK_ERR_INVALID, "tk_topk_backward: bad sizes T=%d E=%d k=%d", n_tokens, n_experts, k);
+  if (n_tokens == 0) return TK_OK;
+  if (!x || !indx || !dy || !dx) return fail(TK_ERR_INVALID, "tk_topk_backward: null pointer");
+  const int rows = n_rows < 0 ? n_tokens : n_rows;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((n_tokens + 3) / 4));
+#define TK_TB(D)                                                                                                                   \
+  if (dtype == D) {                                                                                                                \
+    hipLaunchKernelGGL(topk_backward_kernel<D>, grid, dim3(256), 0, st, x, stride_xm, indx, stride_im, dy, stride_dym, dx, stride_dxm, \
+                       n_tokens, n_experts, k, apply_softmax, rows, n_rows_ptr);                                                   \
+    return check_launch("topk_backward_kernel");                                                                                  \
+  }
+  TK_TB(TK_F32)
+  TK_TB(TK_BF16)
+  TK_TB(TK_F16)
+#undef TK_TB
+  return fail(TK_ERR_UNSUPPORTED, "tk_topk_backward: dtype %d", dtype);
 }

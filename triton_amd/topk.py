@@ -2,8 +2,9 @@
 
 `topk` launches the fused routing pass: selection, gate softmax, bitmatrix, expert histogram and both
 permutations come out of one `tk_route` call, so the returned `SparseMatrix` already carries its
-`mask_metadata`.  The backward pass, `all_gather` and symmetric-memory outputs of the reference are
-training / multi-GPU features and are not part of this build.
+`mask_metadata`.  The backward pass (`topk_backward`, used through autograd when the logits require a gradient)
+is a kernel of its own; `all_gather` and symmetric-memory outputs of the reference are multi-GPU features and are
+not part of this build.
 """
 from __future__ import annotations
 
@@ -59,6 +60,51 @@ def topk_forward(x, k, apply_softmax=True, dim=1, y_indx=None, n_rows=None, all_
     return y_vals, y_indx, mask
 
 
+def topk_backward(x, y_indx, dy_vals, k, n_rows, apply_softmax):
+    """dx [n_tokens, n_expts] for the gradient `dy_vals [n_tokens, k]` of the kept values (topk.py:76-85)."""
+    assert dy_vals.shape[-1] == k and x.ndim == 2
+    nt.require_gpu(x, "x")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    dy = dy_vals.to(x.dtype)
+    if dy.stride(1) != 1:
+        dy = dy.contiguous()
+    indx16 = (y_indx if y_indx.dtype == torch.int16 else y_indx.to(torch.int16)).contiguous()
+    dx = torch.empty_like(x, memory_format=torch.contiguous_format)
+    T, E = x.shape
+    rows_imm, rows_ptr = -1, None
+    if isinstance(n_rows, torch.Tensor):
+        assert n_rows.dtype == torch.int32 and n_rows.is_cuda
+        rows_ptr = n_rows.data_ptr()
+    elif n_rows is not None:
+        rows_imm = int(n_rows)
+    with nt.on_device(x.device):
+        nt.check(
+            nt.lib().tk_topk_backward(x.data_ptr(), nt.TORCH_TO_TK[x.dtype], x.stride(0), indx16.data_ptr(), indx16.stride(0),
+                                      dy.data_ptr(), dy.stride(0), dx.data_ptr(), dx.stride(0), T, E, k, int(bool(apply_softmax)),
+                                      rows_imm, rows_ptr, nt.stream_ptr(x.device)))
+    return dx
+
+
+class TopK(torch.autograd.Function):
+    """Differentiable selection (topk.py:88-105): the gate values carry the gradient; indices, bitmatrix words and
+    metadata are returned as non-differentiable tensors."""
+
+    @staticmethod
+    def forward(ctx, x, k, apply_softmax, y_indx, n_rows):
+        y_vals, indx, mask, r = _topk_route(x.detach(), k, apply_softmax, y_indx, n_rows, want_meta=True)
+        ctx.save_for_backward(x, indx)
+        ctx.k, ctx.apply_softmax, ctx.n_rows = k, apply_softmax, n_rows
+        others = (indx, mask.storage.data, r["col_sum"], r["col_sorted_indx"], r["row_sorted_indx"])
+        ctx.mark_non_differentiable(*others)
+        return (y_vals, *others)
+
+    @staticmethod
+    def backward(ctx, dy_vals, *_unused):
+        x, indx = ctx.saved_tensors
+        return topk_backward(x, indx, dy_vals, ctx.k, ctx.n_rows, ctx.apply_softmax), None, None, None, None
+
+
 def topk(x: Union[Tensor, torch.Tensor], k: int, apply_softmax: bool = True, dim: int = 1,
          y_indx: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, all_gather: bool = False,
          symm_mem_pool=None):
@@ -70,9 +116,13 @@ def topk(x: Union[Tensor, torch.Tensor], k: int, apply_softmax: bool = True, dim
     assert dim == 1
     if all_gather or symm_mem_pool is not None:
         raise NotImplementedError("all_gather / symmetric-memory outputs are multi-GPU features")
-    if x.requires_grad if isinstance(x, torch.Tensor) else False:
-        raise NotImplementedError("topk backward is not part of this build (inference only)")
-    y_vals, y_indx, mask, r = _topk_route(x, k, apply_softmax, y_indx, n_rows, want_meta=True)
+    if isinstance(x, torch.Tensor) and x.requires_grad and torch.is_grad_enabled():
+        y_vals, y_indx, bm_t, col_sum, col_sorted, row_sorted = TopK.apply(x, k, apply_softmax, y_indx, n_rows)
+        T, E = x.shape
+        mask = wrap_torch_tensor(bm_t, dtype=BIT, shape=[T if n_rows is None else n_rows, E], shape_max=[T, None])
+        r = dict(col_sum=col_sum, col_sorted_indx=col_sorted, row_sorted_indx=row_sorted)
+    else:
+        y_vals, y_indx, mask, r = _topk_route(x, k, apply_softmax, y_indx, n_rows, want_meta=True)
     meta = BitmatrixMetadata(col_sum=r["col_sum"], col_sorted_indx=r["col_sorted_indx"],
                              row_sorted_indx=r["row_sorted_indx"])
     return SparseMatrix(vals=y_vals, indx=y_indx, mask=mask, mask_metadata=meta)
