@@ -296,6 +296,14 @@ int32_t tk_reduce_mid(const void* x, int32_t dtype, int64_t A, int64_t K, int64_
                       int64_t ss1, int64_t ss2, void* y, int64_t sy0, tk_stream_t stream);
 
 /*
+ * Replaces `_reduce_backward` (tk/reduce.py:859-1049) for the same subset as tk_reduce_mid: dx [A, K, C] contiguous,
+ * dx[a, j, c] = mask[a, j, c] ? dy[a, c] * scale[a, j, c] : 0, in dy's dtype.
+ */
+int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t K, int64_t C, int64_t sdy0, const void* mask,
+                               int64_t sm0, int64_t sm1, int64_t sm2, const float* scale, int64_t ss0, int64_t ss1, int64_t ss2,
+                               void* dx, tk_stream_t stream);
+
+/*
  * Per-row dynamic quantisation of bf16 activations to OCP e4m3: scales[m] = amax_m / 448 (1 for a zero
  * row), q[m, :] = saturating_cast(x[m, :] / scales[m]).  No counterpart kernel in the reference: its
  * benchmark casts activations to fp8 with a plain torch `.to()` (python/triton_kernels/bench/bench_mlp.py:169);

@@ -80,6 +80,7 @@ SIGNATURES = {
     "tk_moe_gemm": (_i32, [_c.POINTER(GemmDesc), _ptr]),
     "tk_swiglu": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _f32, _f32, _i32, _ptr, _ptr]),
     "tk_reduce_mid": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
+    "tk_reduce_mid_backward": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
     "tk_quant_fp8_rows": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
     "tk_mx_upcast": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i32, _i64, _i64, _i64, _ptr]),
 }

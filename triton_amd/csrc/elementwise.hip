@@ -61,6 +61,22 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const void* x, int64_t 
   }
 }
 
+// Backward of the reduction: dx[a, j, c] = mask[a, j, c] ? dy[a, c] * scale[a, j, c] : 0 (dx contiguous [A, K, C]).
+template <int DT>
+__global__ __launch_bounds__(256) void reduce_mid_backward_kernel(const void* dy, int64_t sdy0, int64_t A, int64_t K, int64_t C,
+                                                                  const uint8_t* mask, int64_t sm0, int64_t sm1, int64_t sm2,
+                                                                  const float* scale, int64_t ss0, int64_t ss1, int64_t ss2, void* dx) {
+  const int64_t total = A * K * C;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t c = i % C, aj = i / C;
+    const int64_t j = aj % K, a = aj / K;
+    float v = ld<DT>(dy, a * sdy0 + c);
+    if (scale) v *= scale[a * ss0 + j * ss1 + c * ss2];
+    if (mask && !mask[a * sm0 + j * sm1 + c * sm2]) v = 0.f;
+    st<DT>(dx, i, v);
+  }
+}
+
 // Fast path of the k-way combine: bf16, no mask / scale, 8 columns (16 bytes) per thread, fp32 sum in j order.
 __global__ __launch_bounds__(256) void reduce_mid_bf16x8_kernel(const uint16_t* x, int64_t sx0, int64_t sx1, int64_t A, int K,
                                                                 int C8, uint16_t* y, int64_t sy0) {
@@ -179,6 +195,26 @@ extern "C" int32_t tk_reduce_mid(const void* x, int32_t dtype, int64_t A, int64_
   else
     return fail(TK_ERR_UNSUPPORTED, "tk_reduce_mid: dtype %d", dtype);
   return check_launch("reduce_mid_kernel");
+}
+
+extern "C" int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t K, int64_t C, int64_t sdy0, const void* mask,
+                                          int64_t sm0, int64_t sm1, int64_t sm2, const float* scale, int64_t ss0, int64_t ss1,
+                                          int64_t ss2, void* dx, tk_stream_t stream) {
+  if (A < 0 || K < 0 || C < 0) return fail(TK_ERR_INVALID, "tk_reduce_mid_backward: negative size");
+  if (A == 0 || K == 0 || C == 0) return TK_OK;
+  if (!dy || !dx) return fail(TK_ERR_INVALID, "tk_reduce_mid_backward: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint8_t* m = static_cast<const uint8_t*>(mask);
+  const int grid = grid_for(A * K * C);
+  if (dtype == TK_BF16)
+    hipLaunchKernelGGL(reduce_mid_backward_kernel<TK_BF16>, dim3(grid), dim3(256), 0, s, dy, sdy0, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, dx);
+  else if (dtype == TK_F16)
+    hipLaunchKernelGGL(reduce_mid_backward_kernel<TK_F16>, dim3(grid), dim3(256), 0, s, dy, sdy0, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, dx);
+  else if (dtype == TK_F32)
+    hipLaunchKernelGGL(reduce_mid_backward_kernel<TK_F32>, dim3(grid), dim3(256), 0, s, dy, sdy0, A, K, C, m, sm0, sm1, sm2, scale, ss0, ss1, ss2, dx);
+  else
+    return fail(TK_ERR_UNSUPPORTED, "tk_reduce_mid_backward: dtype %d", dtype);
+  return check_launch("reduce_mid_backward_kernel");
 }
 
 extern "C" int32_t tk_quant_fp8_rows(const void* x, int32_t dtype, int64_t M, int64_t K, int64_t stride_m, void* q,
