@@ -286,7 +286,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="also run a 1 GiB device copy (reference kernel for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (expert-parallel sharding is described in DESIGN.md)",
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (with more GPUs the layer shards by expert, which is not built)",
               file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
