@@ -32,7 +32,21 @@ def _slice_sizes(m, n_slices, g):
     return sizes.to(torch.int32)
 
 
+_W_CACHE = {}
+
+
 def _make_w(E, K, N, kind, g, device):
+    """Expert weights of one (shape, kind), generated from their own seed and kept for the cases that share them
+    (quantising them with the CPU oracle is the slow part of a case); `g` is left untouched."""
+    key = (E, K, N, kind, str(device))
+    if key not in _W_CACHE:
+        if len(_W_CACHE) >= 6:
+            _W_CACHE.pop(next(iter(_W_CACHE)))
+        _W_CACHE[key] = _make_w_uncached(E, K, N, kind, torch.Generator().manual_seed(E * 1000003 + K * 1009 + N), device)
+    return _W_CACHE[key]
+
+
+def _make_w_uncached(E, K, N, kind, g, device):
     w = (torch.randn((E, K, N), generator=g) * 0.5 / K**0.5 * 4).to(torch.bfloat16)
     if kind in ("mxfp4", "mxfp4_tiled"):
         q, s = omx.downcast_to_mxfp(w, torch.uint8, axis=1)

@@ -70,7 +70,20 @@ def test_config1_small_bf16(api, device):
     assert_allclose_gate(ref, out, what="layer output")
 
 
+_MX_CACHE = {}
+
+
 def _mx_weights(E, d, f2, g, scale=0.02):
+    """MXFP4 expert weights for one shape, from their own seed, quantised once with the CPU oracle (the slow part of
+    a case) and shared by the cases of that shape; `g` is left untouched."""
+    key = (E, d, f2, scale)
+    if key not in _MX_CACHE:
+        _MX_CACHE.clear()
+        _MX_CACHE[key] = _mx_weights_uncached(E, d, f2, torch.Generator().manual_seed(E * 7919 + d + f2), scale)
+    return _MX_CACHE[key]
+
+
+def _mx_weights_uncached(E, d, f2, g, scale=0.02):
     w1 = (torch.randn((E, d, f2), generator=g) * scale).to(torch.bfloat16)
     w2 = (torch.randn((E, f2 // 2, d), generator=g) * scale).to(torch.bfloat16)
     w1q, w1s = omx.downcast_to_mxfp(w1, torch.uint8, axis=1)
