@@ -103,7 +103,8 @@ def downcast_to_mxfp(x: torch.Tensor, out_dtype, axis: int, rounding: int = ROUN
     s = sbits.view(np.float32)
     with np.errstate(divide="ignore"):
         inv = np.where(s == 0, np.float32(0), (np.float32(1.0) / s).astype(np.float32)).astype(np.float32)
-    q = (blocks * inv).astype(np.float32)
+    with np.errstate(invalid="ignore"):  # inf * 0 (an infinite element in a block whose scale overflowed) is NaN on purpose
+        q = (blocks * inv).astype(np.float32)
     scale_bytes = (sbits >> 23).astype(np.uint8).reshape(lead + (L // MX_BLOCK, ))
     if kind == "e2m1":
         codes = e2m1_codes_from_f32(q).reshape(-1, L // 2, 2)
