@@ -1335,7 +1335,6 @@ int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   return check_launch("moe_gemm_mxd_kernel");
 }
 
-// compute units of the current device (cached per device id)
 // Raises a kernel's dynamic LDS limit above 64 KiB, once per device (bit d of `done` = done on device d).  Threads
 // racing through the first call set the same value twice, which is harmless.
 inline int32_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
@@ -1349,6 +1348,7 @@ inline int32_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<uint64
   return TK_OK;
 }
 
+// compute units of the current device (cached per device id)
 inline int device_cu_count() {
   static int cached[64] = {0};
   int dev = 0;
