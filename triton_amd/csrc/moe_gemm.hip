@@ -934,14 +934,15 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 // ------------------------------------------------------------------------------------------------
 // A few rows per expert: the kernel is bound by reading each active expert's weights once.  Every wave works
 // alone (no LDS, no barrier): it owns one 32-column weight fragment of one row block, streams the fragment's
-// K-stages through a four-deep register ring (8 KiB in flight per wave, up to sixteen waves per CU), reads its
-// rows' activations straight from L2 (each lane 64 contiguous bytes per stage), and issues 16x16x32 MFMAs
+// K-stages through a four-deep register ring (8 KiB in flight per wave, twelve to sixteen waves per CU), reads its
+// rows' activations straight from L2 through a ring of the same depth (each lane 64 contiguous bytes per stage;
+// one stage ahead left their latency exposed), and issues 16x16x32 MFMAs
 // transposed like the prefill kernel (lane = column, 4 k-groups).  Within a stage lane group kg owns
 // k in [kg*32, kg*32 + 32): exactly one MX block and one 16-byte piece of the tiled layout.
 template <int MR, bool SWIGLU>
 __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   typedef Frag<16> FR;
-  constexpr int WDD = 4, XDD = 2;  // ring depths (stages) of the weight / activation registers
+  constexpr int WDD = 4, XDD = 4;  // ring depths (stages) of the weight / activation registers (both run 3 stages ahead)
   __shared__ float red[3][2 * MR * 4][64];  // K-split partial sums of waves 1..3
   const int tid = threadIdx.x;
   const int lane = tid & 63;
