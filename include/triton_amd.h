@@ -12,7 +12,8 @@
  *     recorded into a HIP graph;
  *   - scratch memory is supplied by the caller (`workspace` arguments) with the size returned by the
  *     matching *_workspace_bytes function;
- *   - the library keeps no mutable global state apart from the per-thread last-error string.
+ *   - the library's mutable global state is the per-thread last-error string and write-once caches filled
+ *     under a lock or atomically (the compute-unit count per device, which kernels had their LDS limit raised).
  *
  * Each entry point names the reference launch site it replaces; paths are relative to the reference
  * tree root, `python/triton_kernels/triton_kernels/` abbreviated as `tk/`.
@@ -115,7 +116,8 @@ int32_t tk_mx_upcast(const void* vals, const void* scales, int32_t kind, int64_t
  * Selection is a stable descending sort: ties go to the lower expert id; outputs are ordered by value,
  * largest first; the softmax runs over the k kept logits in fp32.  Rows >= n_rows are left untouched
  * in vals / indx / bitmatrix and are not routed.  Optional outputs may be NULL; when col_sum is NULL
- * only the top-k step runs.  Limits: n_experts <= 2048, k <= min(64, n_experts).
+ * only the top-k step runs.  Limits of the entry point: n_experts <= 2048, k <= min(64, n_experts) (the
+ * reference's `topk` is narrower in k: a power of two <= 32, which the Python host enforces).
  */
 typedef struct tk_route_desc {
   const void* logits; /* [n_tokens, n_experts], unit stride along experts; may be NULL with use_provided_indx */
@@ -255,7 +257,7 @@ typedef struct tk_gemm_desc {
   const int32_t* block_offs;     /* [n_slices + 1] for block_m */
   const int32_t* block_schedule; /* [grid_m] for block_m, (block << 16) | slice, -1 padded */
   int32_t n_slices;
-  int32_t block_m; /* 16, 32, 64 or 128 */
+  int32_t block_m; /* 16, 32, 64 or 128; tiled MXFP4 weights also 256; tiled e4m3 weights 128 or 256 only */
   int32_t grid_m;  /* number of row blocks to launch (an upper bound in ragged mode) */
   int32_t M, N, K; /* M: rows of the single slice when not ragged; N: columns of W; K: reduction */
   /* output [rows, N or N/2], unit stride along N */
@@ -266,6 +268,9 @@ typedef struct tk_gemm_desc {
   float act_alpha, act_limit;
   int32_t act_has_limit;
   int32_t w_layout; /* enum tk_w_layout */
+  /* compute units to leave idle: the persistent kernels (tiled weight layouts, block_m >= 64) launch that many
+   * workgroup slots fewer (the reference's `idle_sms`, tk/matmul_details/opt_flags.py:525-529); 0 = use all */
+  int32_t idle_cus;
 } tk_gemm_desc;
 
 /* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */
@@ -311,6 +316,20 @@ int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t
  */
 int32_t tk_quant_fp8_rows(const void* x, int32_t dtype, int64_t M, int64_t K, int64_t stride_m, void* q,
                           int64_t stride_qm, float* scales, tk_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Host check hooks (no device work, no GPU needed)
+ * ---------------------------------------------------------------------------------------------- */
+
+/*
+ * The scalar conversions the MX kernels use, evaluated on the host so that their bit-exactness can be tested on
+ * a machine without a GPU.  tk_host_mx_convert: out[i] = code of in[i] in `kind` (TK_E2M1: 4-bit code in the low
+ * nibble; TK_E4M3 / TK_E5M2: the byte), round to nearest even with saturation.  tk_host_mx_scale: out[i] = e8m0
+ * byte of the block scale for a block whose largest magnitude is absmax[i] (tk/numerics_details/mxfp.py:251-290).
+ * Host pointers.
+ */
+int32_t tk_host_mx_convert(const float* in, int64_t n, int32_t kind, uint8_t* out);
+int32_t tk_host_mx_scale(const float* absmax, int64_t n, int32_t kind, int32_t rounding, uint8_t* out);
 
 #ifdef __cplusplus
 }

@@ -152,3 +152,49 @@ def test_layer_equals_dense_sum_over_selected_experts():
             a = gg * torch.sigmoid(1.3 * gg) * (ll + 1)
             acc += float(vals[t, j]) * (a @ w2[e].double() + b2[e].double())
         assert torch.allclose(out[t].double(), acc, rtol=1e-4, atol=1e-5)
+
+
+def test_layer_gate_against_float64():
+    """How strict the rtol 2e-2 / atol 1e-2 gate is at the LAYER level: the oracle (bf16-rounded intermediates, as the
+    reference materialises them) against an exact float64 evaluation of the same layer on gpt-oss-shaped experts
+    (d 2880, W1 [E, 2880, 5760], W2 [E, 2880, 2880], top-4).  Almost every element is far inside the gate, but not
+    all: the k partial rows are rounded to bf16 before they are summed, so where they cancel the sum carries an
+    absolute error of a partial row's ulp.  This is why the layer-level GPU tests allow a small share of elements
+    outside the gate (LAYER_GATE_SLACK in tests/test_gpu_moe_layer.py) while single GEMMs get none."""
+    g = torch.Generator().manual_seed(2)
+    E, k, d, f2, T = 8, 4, 2880, 5760, 256
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g)
+    # synthetic MXFP4 weights: uniform e2m1 codes with scale 2^-7 have rms 0.023, like N(0, 0.02) weights
+    w1q = torch.randint(0, 256, (E, f2, d // 2), generator=g, dtype=torch.uint8).transpose(1, 2)
+    w2q = torch.randint(0, 256, (E, d, f2 // 4), generator=g, dtype=torch.uint8).transpose(1, 2)
+    w1s = torch.full((E, f2, d // 32), 120, dtype=torch.uint8).transpose(1, 2)
+    w2s = torch.full((E, d, f2 // 64), 120, dtype=torch.uint8).transpose(1, 2)
+    b1 = (torch.randn((E, f2), generator=g) * 0.01).to(torch.bfloat16)
+    b2 = (torch.randn((E, d), generator=g) * 0.01).to(torch.bfloat16)
+    out = omoe.moe_layer(x, logits, k, w1q, b1, w2q, b2, w1_mx_scale=w1s, w2_mx_scale=w2s)
+    W1 = omoe.dequant_weight(w1q, w1s).double()
+    W2 = omoe.dequant_weight(w2q, w2s).double()
+    vals, indx, _ = ort.topk(logits, k)
+    exact = torch.zeros((T, d), dtype=torch.float64)
+    for e in range(E):
+        tj = (indx == e).nonzero()
+        t, j = tj[:, 0], tj[:, 1]
+        h = x[t].double() @ W1[e] + b1[e].double()
+        gg, ll = h[:, ::2].clamp(max=7.0), h[:, 1::2].clamp(-7.0, 7.0)
+        a = gg * torch.sigmoid(1.702 * gg) * (ll + 1)
+        exact.index_add_(0, t, (a @ W2[e] + b2[e].double()) * vals[t, j].double()[:, None])
+    err = (out.double() - exact).abs()
+    outside = err > (1e-2 + 2e-2 * exact.abs())
+    frac = float(outside.double().mean())
+    print(f"oracle vs float64: worst |err| {float(err.max()):.4g}, median {float(err.median()):.4g}, output rms "
+          f"{float(exact.pow(2).mean().sqrt()):.4g}, outside the gate {int(outside.sum())} of {outside.numel()}")
+    # the worst element sits at the gate (an ulp of a partial row) while the typical one is far inside it
+    assert float(err.max()) > 5e-3, f"worst error {float(err.max()):.3g}: the gate would be loose here"
+    assert float(err.median()) < 0.2 * float(err.max())
+    # the oracle itself is outside the gate for about two elements in 100 000 here: a zero-tolerance gate at layer
+    # level would reject the oracle; the GPU tests allow 1e-4
+    assert int(outside.sum()) > 0 and frac <= 1e-4, f"{frac:.3g} of the oracle's own elements are outside the gate"
+    # rounding the exact result once to bf16 is always inside the gate: the slack comes from the partial rows
+    once = (exact.to(torch.bfloat16).double() - exact).abs() > (1e-2 + 2e-2 * exact.abs())
+    assert int(once.sum()) == 0

@@ -63,7 +63,7 @@ class GemmDesc(_c.Structure):
         ("n_slices", _i32), ("block_m", _i32), ("grid_m", _i32), ("M", _i32), ("N", _i32), ("K", _i32),
         ("y", _ptr), ("y_dtype", _i32), ("y_stride_m", _i64),
         ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
-        ("w_layout", _i32),
+        ("w_layout", _i32), ("idle_cus", _i32),
     ]
 
 
@@ -83,10 +83,7 @@ SIGNATURES = {
     "tk_reduce_mid_backward": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
     "tk_quant_fp8_rows": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
     "tk_mx_upcast": (_i32, [_ptr, _ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i32, _i64, _i64, _i64, _ptr]),
-}
-
-# host-side check hooks (not part of the device ABI)
-HOST_SIGNATURES = {
+    # host check hooks (no device work)
     "tk_host_mx_convert": (_i32, [_ptr, _i64, _i32, _ptr]),
     "tk_host_mx_scale": (_i32, [_ptr, _i64, _i32, _i32, _ptr]),
 }
@@ -110,7 +107,7 @@ def lib():
                         f"{LIB_PATH} not found: build it with `python -m triton_amd.build` (needs hipcc). "
                         "There is no fallback implementation.")
                 handle = ctypes.CDLL(LIB_PATH)
-                for name, (res, args) in {**SIGNATURES, **HOST_SIGNATURES}.items():
+                for name, (res, args) in SIGNATURES.items():
                     fn = getattr(handle, name)
                     fn.restype = res
                     fn.argtypes = args

@@ -20,7 +20,9 @@
 //   * the rows of a tile are dealt to the WM row-waves in interleaved 16-row fragments and fragments
 //     past the expert's last row are skipped, so a nearly empty row block costs almost no MFMA time.
 #include <atomic>
+#include <mutex>
 #include <type_traits>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -79,6 +81,7 @@ struct GemmParams {
   int32_t bias_vec;  // bias rows allow 16-byte vector loads
   int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
   int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
+  int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
 };
 
 __device__ inline int xcd_remap(int pid, int total) {
@@ -1336,30 +1339,46 @@ int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   return check_launch("moe_gemm_mxd_kernel");
 }
 
-// Raises a kernel's dynamic LDS limit above 64 KiB, once per device (bit d of `done` = done on device d).  Threads
-// racing through the first call set the same value twice, which is harmless.
-inline int32_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
+// Raises a kernel's dynamic LDS limit above 64 KiB, once per (kernel, device): the table is keyed on the kernel's
+// address, so every template instantiation (the swiglu and the plain variant of one tile shape included) has an
+// entry of its own; bit d of an entry = done on device d.
+inline int32_t allow_dynamic_lds(const void* kern, int bytes) {
   if (bytes <= 64 * 1024) return TK_OK;
+  static std::mutex mu;
+  static std::unordered_map<const void*, uint64_t> done;
   int dev = 0;
   const bool known = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64;
-  if (known && (done.load(std::memory_order_acquire) >> dev & 1ull)) return TK_OK;
+  if (known) {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = done.find(kern);
+    if (it != done.end() && (it->second >> dev & 1ull)) return TK_OK;
+  }
   hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
-  if (known) done.fetch_or(1ull << dev, std::memory_order_release);
+  if (known) {
+    std::lock_guard<std::mutex> lock(mu);
+    done[kern] |= 1ull << dev;
+  }
   return TK_OK;
 }
 
-// compute units of the current device (cached per device id)
+// compute units of the current device (cached per device id; racing first calls store the same value)
 inline int device_cu_count() {
-  static int cached[64] = {0};
+  static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
+}
+
+// compute units a persistent grid may fill when `idle` of them are to stay free (at least one is used)
+inline int busy_cu_count(int idle) {
+  const int n = device_cu_count() - (idle > 0 ? idle : 0);
+  return n > 0 ? n : 1;
 }
 
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD>
@@ -1373,11 +1392,10 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   q.total_tiles = (int32_t)grid;
   // persistent grid: as many workgroups as fit on the device at once (LDS decides how many share a CU)
   const int per_cu = LDS_BYTES > 80 * 1024 ? 1 : 2;
-  const int64_t resident = (int64_t)device_cu_count() * per_cu;
+  const int64_t resident = (int64_t)busy_cu_count(p.idle_cus) * per_cu;
   if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
-    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
-    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256 * G), LDS_BYTES, st, q);
     return check_launch("moe_gemm_mxn_kernel");
   };
@@ -1395,11 +1413,10 @@ int32_t launch_f8n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   q.total_tiles = (int32_t)grid;
   // persistent grid, one workgroup per CU (the register ring and the accumulators take a wave's whole budget)
-  const int64_t resident = (int64_t)device_cu_count();
+  const int64_t resident = (int64_t)busy_cu_count(p.idle_cus);
   if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
-    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
-    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
     return check_launch("moe_gemm_f8n_kernel");
   };
@@ -1420,8 +1437,7 @@ int32_t launch_cfg(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   auto launch = [&](auto kern) -> int32_t {
-    static std::atomic<uint64_t> lds_allowed{0};  // one flag set per kernel instantiation
-    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, lds_allowed)) return rc;
+    if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), LDS_BYTES, st, q);
     return check_launch("moe_gemm_kernel");
   };
@@ -1526,6 +1542,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.y_vec = (d->y_stride_m % 8 == 0) && ((reinterpret_cast<uintptr_t>(d->y) & 15) == 0);
   p.bias_vec = d->bias && (d->bias_stride_e % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->bias) & 15) == 0);
   p.grid_n = 0;
+  p.idle_cus = d->idle_cus;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
   if (d->w_layout == TK_W_TILED && d->w_dtype == TK_E4M3) {

@@ -7,7 +7,7 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
 
     activations  weights                        notes
     bf16         bf16                           K-contiguous weights are used in place; N-contiguous
-                                                ones are re-laid out once per call
+                                                ones are re-laid out once (the copy is cached on the tensor)
     bf16         mxfp4 (uint8 e2m1 + e8m0)      dequantised in registers, bf16 MFMA, fp32 accumulate
     fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
 
@@ -108,10 +108,22 @@ def _flex_out_is_trivial(flex: FlexCtx) -> bool:
 
 
 def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
-    """[E, K, N] weights with unit stride along K (each output column contiguous in memory)."""
+    """[E, K, N] weights with unit stride along K (each output column contiguous in memory).  Weights that arrive
+    N-contiguous (a plain torch [E, K, N] tensor) are re-laid out ONCE: the copy is kept on the tensor object,
+    keyed by the tensor's version counter so that an in-place update of the weights makes a new copy.  The copy
+    doubles the memory of such weights; callers that mind convert them up front (`w.transpose(-1, -2).contiguous()
+    .transpose(-1, -2)`, or `convert_layout(w, StridedLayout(-2))`) and drop the original."""
     if w.stride(-2) == 1 and (w.shape[-2] == 1 or w.stride(-1) >= w.shape[-2]):
         return w
-    return w.transpose(-1, -2).contiguous().transpose(-1, -2)
+    cached = getattr(w, "_tk_k_contiguous", None)
+    if cached is not None and cached[0] == w._version:
+        return cached[1]
+    conv = w.transpose(-1, -2).contiguous().transpose(-1, -2)
+    try:
+        w._tk_k_contiguous = (w._version, conv)
+    except (AttributeError, RuntimeError):
+        pass  # a tensor subclass without a __dict__: converted per call
+    return conv
 
 
 def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
@@ -247,6 +259,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         assert precision_config.b_microblock_size is None or precision_config.b_microblock_size == MXFP_BLOCK_SIZE, \
             f"Unsupported microscale block size {precision_config.b_microblock_size}"
     w = b.storage.data
+    if not tiled and not tiled_fp8 and b.dtype != FP4:
+        w = _k_contiguous(w)  # before any view is taken: the converted copy is cached on the caller's tensor
     if w.ndim == 2 and not tiled and not tiled_fp8:
         w = w[None]
     K_W, N = b.shape[-2:]
@@ -329,9 +343,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         assert w.dtype == torch.uint8
         if w.stride(-2) != 1:
             raise NotImplementedError("mxfp4 weights must be packed along K (stride(-2) == 1)")
-        ws = b_scale.storage.data
+        ws = _k_contiguous(b_scale.storage.data)
         ws = ws[None] if ws.ndim == 2 else ws
-        ws = _k_contiguous(ws)
         d.w_dtype = nt.TK_E2M1
         d.w_mx_scale = ws.data_ptr()
         d.ws_stride_e, d.ws_stride_k, d.ws_stride_n = ws.stride()
@@ -339,7 +352,6 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     else:
         if b_scale is not None:
             raise NotImplementedError("MX scales are supported with mxfp4 (uint8) weights only")
-        w = _k_contiguous(w)
         d.w_dtype = nt.TORCH_TO_TK.get(w.dtype, -1)
     d.w = w.data_ptr()
     if tiled or tiled_fp8:
@@ -413,6 +425,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.y_stride_m = c.stride(0)
     d.activation = act
     d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
+    d.idle_cus = max(0, int(opt_flags.idle_sms or 0))
     with nt.on_device(a.device):
         nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
     del keep

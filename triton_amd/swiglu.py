@@ -50,7 +50,11 @@ def swiglu(a, alpha, precision_config, routing_data=None):
     out = torch.empty((M, N // 2), dtype=a.dtype, device=a.device)
     n_tokens = None
     if routing_data is not None:
-        n_tokens = routing_data.expt_data.token_offs[routing_data.n_expts_tot:routing_data.n_expts_tot + 1]
+        # rows actually routed = the last entry of the experts' row offsets (the reference reads
+        # `expt_data.token_offs[n_expts_tot]`, swiglu.py:53-55; here the same array is called `slice_offs`)
+        offs = routing_data.expt_data.slice_offs
+        n_tokens = offs[routing_data.n_expts_tot:routing_data.n_expts_tot + 1]
+        assert n_tokens.dtype == torch.int32 and n_tokens.numel() == 1
     limit = precision_config.limit
     with nt.on_device(a.device):
         nt.check(
