@@ -11,9 +11,10 @@
  *     kernels on `stream` (a hipStream_t passed as void*), so every call is stream-ordered and can be
  *     recorded into a HIP graph;
  *   - scratch memory is supplied by the caller (`workspace` arguments) with the size returned by the
- *     matching *_workspace_bytes function;
+ *     matching *_workspace_bytes function (tk_route_static, which owns its scratch, is the one exception);
  *   - the library's mutable global state is the per-thread last-error string and write-once caches filled
- *     under a lock or atomically (the compute-unit count per device, which kernels had their LDS limit raised).
+ *     under a lock or atomically (the compute-unit count per device, which kernels had their LDS limit raised,
+ *     the device address of tk_route_static's scratch array).
  *
  * Each entry point names the reference launch site it replaces; paths are relative to the reference
  * tree root, `python/triton_kernels/triton_kernels/` abbreviated as `tk/`.
@@ -152,6 +153,19 @@ typedef struct tk_route_desc {
 
 int64_t tk_route_workspace_bytes(int32_t n_tokens, int32_t n_experts);
 int32_t tk_route(const tk_route_desc* desc, tk_stream_t stream);
+
+/*
+ * tk_route for callers that cannot allocate.  No counterpart in the reference: it is for code under HIP graph
+ * capture, tight serving loops and harnesses that forbid hipMalloc, which cannot provide `workspace`.  Same
+ * arguments and results as tk_route, except that `desc->workspace` is ignored: the kernels' scratch memory is a
+ * device array inside the library (TK_ROUTE_STATIC_SCRATCH_BYTES per GPU, held until the process ends), so the
+ * call allocates nothing.  Problems with tk_route_workspace_bytes(n_tokens, n_experts) above that size are
+ * refused with TK_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (different streams, different threads) race and must be serialised by the caller; calls in stream order are
+ * safe, the array's previous contents are never read.
+ */
+#define TK_ROUTE_STATIC_SCRATCH_BYTES (2 * 1024 * 1024)
+int32_t tk_route_static(const tk_route_desc* desc, tk_stream_t stream);
 
 /*
  * Replaces `_topk_backward` (tk/topk_details/_topk_backward.py:5-51, launched by tk/topk.py:76-85): gradient of the

@@ -16,6 +16,8 @@
 //   route_scatter_kernel each wave re-reads its tokens' expert ids in flat (token-major) order, ranks
 //                        equal ids with ballots (stable), and writes both permutations plus the
 //                        optional gather index / gate value in expert-sorted order.
+#include <mutex>
+
 #include "common.h"
 
 namespace tk {
@@ -803,8 +805,9 @@ extern "C" int64_t tk_route_workspace_bytes(int32_t T, int32_t E) {
   return (units_pad * E + (int64_t)E + 1) * 4;
 }
 
-extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
-  if (!d) return fail(TK_ERR_INVALID, "tk_route: null descriptor");
+// One routing pass with the kernels' scratch memory at `workspace` (tk_route_workspace_bytes(T, E) bytes, every word
+// of which is written before it is read, so the memory may hold anything).
+static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t stream) {
   const int T = d->n_tokens, E = d->n_experts, k = d->k;
   if (T < 0 || E <= 0 || k <= 0) return fail(TK_ERR_INVALID, "tk_route: bad sizes T=%d E=%d k=%d", T, E, k);
   if (k > 64 || k > E) return fail(TK_ERR_INVALID, "tk_route: k=%d must be <= min(64, E)", k);
@@ -813,13 +816,13 @@ extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
   const bool want_meta = d->col_sum != nullptr;
   if (!d->indx) return fail(TK_ERR_INVALID, "tk_route: indx buffer is required");
   if (!d->logits && !d->use_provided_indx) return fail(TK_ERR_INVALID, "tk_route: logits are required unless indices are provided");
-  if (want_meta && (!d->col_sorted_indx || !d->row_sorted_indx || !d->workspace)) return fail(TK_ERR_INVALID, "tk_route: metadata outputs / workspace missing");
+  if (want_meta && (!d->col_sorted_indx || !d->row_sorted_indx || !workspace)) return fail(TK_ERR_INVALID, "tk_route: metadata outputs / workspace missing");
   if (d->indx_dtype != TK_I16) return fail(TK_ERR_UNSUPPORTED, "tk_route: indx must be int16");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int rpw = rows_per_wave_for(T);
   const int units = (T + rpw - 1) / rpw;
   const int units_pad = (units + kWaves - 1) / kWaves * kWaves;
-  int32_t* partials = static_cast<int32_t*>(d->workspace);
+  int32_t* partials = static_cast<int32_t*>(workspace);
   int32_t* col_offs = partials ? partials + (int64_t)units_pad * E : nullptr;
 
   TopkParams tp;
@@ -908,6 +911,48 @@ extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
   sp.vals_bytes = (d->logits_dtype == TK_F32 || !d->logits) ? 4 : 2;
   hipLaunchKernelGGL(route_scatter_kernel, dim3(units_pad / kWaves), dim3(kWaves * 64), 0, st, sp);
   return check_launch("route_scatter_kernel");
+}
+
+extern "C" int32_t tk_route(const tk_route_desc* d, tk_stream_t stream) {
+  if (!d) return fail(TK_ERR_INVALID, "tk_route: null descriptor");
+  return route_impl(d, d->workspace, stream);
+}
+
+// ---- routing without any allocation: the workspace is a device array owned by the library ------------------
+// `route_scratch` exists once per GPU the library runs on and lives until the process ends.  Host code never
+// passes the array's name to a kernel (on the host it is a stand-in, not a device address): the address on the
+// current device is looked up once per device with hipGetSymbolAddress and kept in `g_route_scratch`.
+constexpr int64_t kRouteScratchBytes = TK_ROUTE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char route_scratch[kRouteScratchBytes];
+
+static std::mutex g_route_scratch_mu;
+static void* g_route_scratch[64];  // per device id, filled under the mutex
+
+static int32_t route_scratch_ptr(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "tk_route_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= 64) return fail(TK_ERR_UNSUPPORTED, "tk_route_static: device id %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_route_scratch_mu);
+  if (!g_route_scratch[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(route_scratch));
+    if (e != hipSuccess || !ptr) return fail(TK_ERR_LAUNCH, "tk_route_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_route_scratch[dev] = ptr;
+  }
+  *out = g_route_scratch[dev];
+  return TK_OK;
+}
+
+extern "C" int32_t tk_route_static(const tk_route_desc* d, tk_stream_t stream) {
+  if (!d) return fail(TK_ERR_INVALID, "tk_route_static: null descriptor");
+  const int64_t need = tk_route_workspace_bytes(d->n_tokens, d->n_experts);
+  if (need > kRouteScratchBytes)
+    return fail(TK_ERR_UNSUPPORTED, "tk_route_static: %d tokens x %d experts need %lld bytes of scratch, the built-in buffer holds %lld; use tk_route with a caller workspace",
+                d->n_tokens, d->n_experts, (long long)need, (long long)kRouteScratchBytes);
+  void* ws = nullptr;
+  if (const int32_t rc = route_scratch_ptr(&ws)) return rc;
+  return route_impl(d, ws, stream);
 }
 
 extern "C" int32_t tk_ragged_metadata(const int32_t* slice_sizes, int32_t n_slices, int32_t* slice_offs, int32_t* block_offs,

@@ -26,8 +26,10 @@ class BitmatrixMetadata:
 
 
 def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_indx, vals, bitmatrix_data, want_meta,
-           want_extras=False, ragged=None):
-    """Fills and submits a tk_route_desc.  Returns a dict of the tensors it allocated."""
+           want_extras=False, ragged=None, static_scratch=False):
+    """Fills and submits a tk_route_desc.  Returns a dict of the tensors it allocated.  With `static_scratch` the
+    kernels' workspace is the library's own device array (`tk_route_static`) instead of a part of the allocation
+    made here."""
     dev = indx16.device
     T = indx16.shape[0]
     R = T * k
@@ -58,7 +60,7 @@ def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_
         # one int32 allocation carved into the histogram, both permutations (adjacent, as the reference carves them
         # from one [2R] buffer, bitmatrix.py:119-121), the gather index and the kernels' workspace
         e_pad = (n_experts + 3) & ~3
-        ws_words = (max(1, nt.lib().tk_route_workspace_bytes(T, n_experts)) + 3) // 4
+        ws_words = 0 if static_scratch else (max(1, nt.lib().tk_route_workspace_bytes(T, n_experts)) + 3) // 4
         r_pad = (R + 3) & ~3
         n_gather = r_pad if want_extras else 0
         buf = torch.empty((e_pad + 2 * r_pad + n_gather + ws_words, ), dtype=torch.int32, device=dev)
@@ -69,7 +71,7 @@ def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_
         d.col_sum = col_sum.data_ptr()
         d.col_sorted_indx = combined.data_ptr()
         d.row_sorted_indx = combined.data_ptr() + 4 * R
-        d.workspace = ws.data_ptr()
+        d.workspace = None if static_scratch else ws.data_ptr()
         if want_extras:
             gather = buf[e_pad + 2 * r_pad:e_pad + 2 * r_pad + R]
             d.gather_indx = gather.data_ptr()
@@ -88,7 +90,8 @@ def _route(logits, indx16, n_rows, n_experts, k, *, apply_softmax, use_provided_
             d.max_n_blocks = width
     if T > 0:
         with nt.on_device(dev):
-            nt.check(nt.lib().tk_route(d, nt.stream_ptr(dev)))
+            entry = nt.lib().tk_route_static if static_scratch else nt.lib().tk_route
+            nt.check(entry(d, nt.stream_ptr(dev)))
     elif want_meta:
         out["col_sum"].zero_()
     return out
