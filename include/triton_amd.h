@@ -215,6 +215,9 @@ int32_t tk_ragged_remap(const int32_t* slice_sizes, const int32_t* slice_offs, c
  *           k in [s*128 + h*64 + q*32, +32);
  *   scales  one 128-byte block at ((F * S + s) * 128) ordered [c:32][4]: the four e8m0 bytes of column
  *           F*32 + c for the stage's four 32-element blocks.
+ * With this layout and block_m >= 64: at most 1024 slices; x and y each span less than 4 GiB / 2 GiB; output rows are
+ * 16-byte aligned with a row stride of at least N_out rounded up to 8 (whole 16-byte pieces are written, the
+ * padding columns receive unspecified values); x_row_scale / w_col_scale are not supported.
  * With w_dtype == TK_E4M3 (e4m3 activations, no MX scales) TK_W_TILED is the one-byte variant of the same idea:
  *   values  K padded to 256 (S = 2 * ceil(K / 256) blocks of 128 per fragment); one 4096-byte block at
  *           ((F * S + s) * 4096) ordered [q:4][lane:64][16 bytes]; lane = h*32 + c holds
@@ -285,7 +288,19 @@ typedef struct tk_gemm_desc {
   /* compute units to leave idle: the persistent kernels (tiled weight layouts, block_m >= 64) launch that many
    * workgroup slots fewer (the reference's `idle_sms`, tk/matmul_details/opt_flags.py:525-529); 0 = use all */
   int32_t idle_cus;
+  /* Optional scratch for the persistent kernels: TK_GEMM_TILE_COUNTER_WORDS int32 words, zero before the first
+   * launch that uses them.  With it, and when the tiles do not divide evenly among the workgroups, a workgroup
+   * takes its first two tiles from a fixed schedule and claims the following ones with atomic counters (one queue
+   * per XCD), which evens out tiles of different cost; the kernel leaves the words zero again, so one buffer serves
+   * any number of launches in stream order, but launches that may overlap in time (other streams) need their own
+   * words.  NULL = fixed schedule.  No counterpart in the reference (its AMD path is not persistent). */
+  int32_t* tile_counters;
+  /* rows of x (with gather_indx: every index is below it); 0 = not stated (then M when not gathering).  The kernels
+   * for tiled MXFP4 weights at block_m >= 64 need x to span less than 4 GiB and refuse larger ones. */
+  int64_t x_rows;
 } tk_gemm_desc;
+
+#define TK_GEMM_TILE_COUNTER_WORDS 16
 
 /* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */
 int32_t tk_moe_gemm(const tk_gemm_desc* desc, tk_stream_t stream);

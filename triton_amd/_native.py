@@ -63,7 +63,7 @@ class GemmDesc(_c.Structure):
         ("n_slices", _i32), ("block_m", _i32), ("grid_m", _i32), ("M", _i32), ("N", _i32), ("K", _i32),
         ("y", _ptr), ("y_dtype", _i32), ("y_stride_m", _i64),
         ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
-        ("w_layout", _i32), ("idle_cus", _i32),
+        ("w_layout", _i32), ("idle_cus", _i32), ("tile_counters", _ptr), ("x_rows", _i64),
     ]
 
 

@@ -82,6 +82,81 @@ struct GemmParams {
   int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
   int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
   int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
+  int32_t* tile_counters;  // persistent kernels: kTileCounterWords zeroed words for dynamic tile claiming, or null
+  uint32_t y_bytes;        // persistent MXFP4 kernels: bytes of the output buffer that rows may be written to (< 2 GiB)
+};
+
+// Persistent kernels hand out tiles either statically (round r gives workgroup b tile r * grid + remap(b)) or, when the
+// caller supplies `tile_counters`, dynamically: the tile list is cut into 8 contiguous queues, one per XCD, and a
+// workgroup claims the next tile of its XCD's queue with an atomic increment (tiles that share weights or
+// activations keep running next to each other under one L2); when its queue is empty it takes from the other
+// queues in ring order.  Tiles cost different amounts (4 or 5 row fragments, partly filled column tiles), so a
+// static deal waits for the slowest tile of every round.  The claim for the NEXT tile is issued when a tile starts and
+// read when it ends, so the atomic's latency is hidden behind the tile's K loop.  Words 0..7 = next index of each
+// queue, word 8 = workgroups that have finished; the last one to finish clears all nine words, so the counters
+// are zero again when the kernel ends (launches that share the words must not overlap in time).
+constexpr int kTileCounterWords = 16;
+
+struct TileClaimer {
+  int32_t* ctr;
+  int live;
+  int myq;
+  int pending;   // thread 0: index returned by the claim in flight
+  __device__ __forceinline__ int qbeg(int q) const { return (int)(((int64_t)live * q) >> 3); }
+  // Workgroups that start on queue q number ((grid - q + 7) / 8); each takes two tiles of the queue without asking
+  // (indices blockIdx.x / 8 and that plus their number), so the counters count from twice their number.
+  __device__ __forceinline__ int qwgs(int q) const { return ((int)gridDim.x - q + 7) >> 3; }
+  __device__ __forceinline__ int qfirst(int q) const { return 2 * qwgs(q); }
+  // second tile of this workgroup (thread-uniform, no memory access), -1 if its queue is shorter than that
+  __device__ __forceinline__ int second() const {
+    const int t = qbeg(myq) + (int)(blockIdx.x >> 3) + qwgs(myq);
+    return t < qbeg(myq + 1) ? t : -1;
+  }
+  // first tile of this workgroup (thread-uniform, no memory access), -1 if its queue is shorter than that
+  __device__ __forceinline__ int init(int32_t* c, int live_tiles) {
+    ctr = c;
+    live = live_tiles;
+    myq = blockIdx.x & 7;
+    pending = 0;
+    const int t = qbeg(myq) + (int)(blockIdx.x >> 3);
+    return t < qbeg(myq + 1) ? t : -1;
+  }
+  // thread 0: start the claim of this workgroup's next tile (own queue)
+  // (the result goes through a variable that is undefined in the other lanes: merging it with the previous value
+  // would make every lane wait for the atomic to return right here)
+  __device__ __forceinline__ void issue() {
+    int fresh;
+    if (threadIdx.x == 0) fresh = atomicAdd(&ctr[myq], 1);
+    pending = fresh;
+  }
+  // thread 0: tile id of the claim in flight, or of another queue when the own one is exhausted; -1 = no tile left.
+  // The other queues' counters are read together first, so a workgroup that finds everything taken pays two
+  // memory round trips, not eight.
+  __device__ __forceinline__ int resolve() {
+    int t = qbeg(myq) + qfirst(myq) + pending;
+    if (t < qbeg(myq + 1)) return t;
+    int seen[8];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) seen[i] = __hip_atomic_load(&ctr[(myq + i) & 7], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      const int q = (myq + i) & 7;
+      if (qbeg(q) + qfirst(q) + seen[i] >= qbeg(q + 1)) continue;  // counters only grow: taken stays taken
+      t = qbeg(q) + qfirst(q) + atomicAdd(&ctr[q], 1);
+      if (t < qbeg(q + 1)) return t;
+    }
+    return -1;
+  }
+  // thread 0, once, after the workgroup's last claim: count it as finished; the last workgroup clears the counters
+  __device__ __forceinline__ void finish() {
+    if (threadIdx.x == 0) {
+      __threadfence();
+      if (atomicAdd(&ctr[8], 1) == (int)gridDim.x - 1) {
+        __threadfence();
+        for (int i = 0; i < 9; ++i) atomicExch(&ctr[i], 0);
+      }
+    }
+  }
 };
 
 __device__ inline int xcd_remap(int pid, int total) {
@@ -646,15 +721,89 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 // BLKM = rows of a row block in the ragged metadata (block_m).  A tile processes its block in passes of
 // BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 5 an expert of up to 160 rows is ONE tile (weights read
 // once, no nearly empty second tile) and only larger blocks take a second pass.
+// Slices (experts) whose row and block offsets the persistent MXFP4 prefill kernel keeps in LDS: a tile's coordinates
+// then cost LDS reads instead of a chain of dependent global loads.  The host refuses more slices than this.
+constexpr int kMetaSlices = 1024;
+
+// Epilogue of the persistent prefill kernels.  Everything a tile's rows and columns need (bias as fp32, gate weight,
+// destination row or -1) was fetched ahead and sits in LDS: bias_s[BN] by tile column, gam_s / dst_s [BM] by tile
+// row.  Order: bias, activation, gate weight, (scattered) store.  The bias is added as each accumulator register
+// is read for the last time (a pass of its own over the accumulators would move all of them between the
+// accumulation and the vector registers twice more).
+// Every lane executes every store instruction: rows without a destination and columns past N get a byte offset
+// beyond the buffer resource's range, which the hardware drops.  With no branch around a store the number of
+// stores between two loads is the same on every path, so the compiler's vmcnt waits for loads issued BEFORE the
+// epilogue (the next unit's first operands) do not wait for these stores to drain.
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+constexpr uint32_t kDroppedStore = 0x80000000u;  // output buffers span less than 2 GiB (checked by the host)
+
+template <int G, int MFW, int NFW, bool SWIGLU>
+__device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc, const float* bias_s,
+                                                const float* gam_s, const int* dst_s, int ncol_tile, int ncol0, int grp, int lr, int h) {
+  const int NOUT = SWIGLU ? p.N / 2 : p.N;
+  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
+  const float limit = p.has_limit ? p.limit : INFINITY;
+  const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const int r = (j * G + grp) * 32 + lr;
+    const float g = gam_s[r];
+    const int dst = dst_s[r];
+    const uint32_t row_off = dst >= 0 ? (uint32_t)dst * row_bytes : kDroppedStore;
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i: after the two
+        // lane halves exchange their 4-column groups a lane holds 8 consecutive columns from 16u + 8h
+        float v[8];
+        // bias of the two column groups (zeros without a bias), re-read from LDS for every row fragment: keeping all
+        // of a lane's 32 bias values in registers costs more than the reads
+        const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 4 * h);
+        const f32x4_t b1 = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 8 + 4 * h);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          uint32_t lo = f32_bits(acc[f][j][8 * u + i] + b0[i]), hi = f32_bits(acc[f][j][8 * u + 4 + i] + b1[i]);
+          auto sw = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);
+          v[i] = bits_f32(sw[0]);
+          v[4 + i] = bits_f32(sw[1]);
+        }
+        const int n0 = ncol0 + f * 32 + 16 * u + 8 * h;  // first of this lane's 8 columns
+        if (SWIGLU) {
+          float o[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[i] = swiglu_f(v[2 * i], v[2 * i + 1], nalpha_log2e, limit) * g;
+          const int o0 = n0 / 2;
+          const uint32_t off = (o0 < NOUT && dst >= 0) ? row_off + (uint32_t)o0 * 2u : kDroppedStore;
+          const u32x2_t w = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+          __builtin_amdgcn_raw_buffer_store_b64(w, yrsrc, off, 0, 0);
+        } else {
+          const uint32_t off = (n0 < NOUT && dst >= 0) ? row_off + (uint32_t)n0 * 2u : kDroppedStore;
+          u32x4_t w;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i] * g, v[2 * i + 1] * g);
+          __builtin_amdgcn_raw_buffer_store_b128(w, yrsrc, off, 0, 0);
+        }
+      }
+  }
+}
+
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD, bool SWIGLU>
 __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams p) {
   typedef Frag<32> FR;
   constexpr int FM = 32, NT = 256 * G, BM = MFW * 32 * G, BN = 128 * NFW, KC = 128;
   static_assert((WD == 2 || WD == 4) && (XD == 1 || XD == 2), "ring depths");
+  static_assert(BM <= NT && BN <= NT, "one thread per tile row and per tile column fetches the epilogue operands");
   constexpr int XPITCH = KC * 2 + 16;
   constexpr int XBYTES = BM * XPITCH;
   constexpr int XCH = BM * 16 / NT;  // 16-byte activation pieces per thread per stage (4 or 8)
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int32_t soffs_s[kMetaSlices], ssize_s[kMetaSlices], boffs_s[kMetaSlices + 1];
+  // per-unit operands, two sets used in turn: set (u & 1) holds unit u's epilogue operands and unit u+1's gather indices
+  __shared__ __attribute__((aligned(16))) float bias_s[2][BN];
+  __shared__ float gam_s[2][BM];
+  __shared__ int32_t dst_s[2][BM], gidx_s[2][BM];
+  __shared__ int next_tile_s[2];  // slot (n & 1): id of the tile after the next, written during this workgroup's n-th tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -663,73 +812,167 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   const int lr = lane & 31, h = lane >> 5;
   const int K = p.K, N = p.N;
   const int nst = p.w_nst;
-  // Persistent workgroups: the grid is a few workgroups per CU and each walks over tiles round by round, so
-  // no CU waits for the dispatcher between tiles.  A round is gridDim.x consecutive tile ids; inside a round
-  // the ids are dealt so that each XCD (which receives every 8th workgroup) works on a contiguous run.
-  const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
-  for (int round0 = 0; round0 < live; round0 += (int)gridDim.x) {
-  const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
-  if ((int)blockIdx.x >= in_round) break;
-  const int pid = round0 + xcd_remap(blockIdx.x, in_round);
-  int expert, off_m, start_m, eM, pid_n;
-  if (p.slice_sizes) {
-    // Tiles are ordered (expert, column tile, row block): the row blocks of one expert that share a column
-    // tile get consecutive ids, run at the same time on one XCD and stream the same weights through its L2.
-    expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
-    const int first = p.block_offs[expert];
-    const int nb = p.block_offs[expert + 1] - first;
-    const int local = pid - first * p.grid_n;
-    pid_n = local / nb;
-    off_m = (local - pid_n * nb) * BLKM;
-    start_m = p.slice_offs[expert];
-    eM = p.slice_sizes[expert];
-  } else {
-    pid_n = pid % p.grid_n;
-    expert = 0;
-    off_m = (pid / p.grid_n) * BLKM;
-    start_m = 0;
-    eM = p.M;
-  }
-  const int blk_off = off_m;
-  const int blk_rows = (eM - blk_off) < BLKM ? (eM - blk_off) : BLKM;
-  for (int pass_off = 0; pass_off < blk_rows; pass_off += BM) {
-  const int off_m = blk_off + pass_off;
-  const int rows = (blk_rows - pass_off) < BM ? (blk_rows - pass_off) : BM;
-  const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW*G)
-
-  // ---- activation staging: this thread's 16-byte pieces (row r_j = tid/16 + 16 j, k-chunk c = tid%16) ----
-  const int xc = tid & 15;
-  const uint8_t* xptr[XCH];
-#pragma unroll
-  for (int j = 0; j < XCH; ++j) {
-    const int r = (tid >> 4) + (NT / 16) * j;
-    int row = off_m + r;
-    row = row < eM ? row : eM - 1;
-    const int64_t src = p.gather ? (int64_t)p.gather[start_m + row] : (int64_t)(start_m + row);
-    xptr[j] = p.x + src * p.x_stride_m * 2;  // the k offset (incl. this thread's chunk) is added per stage
-  }
-  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // piece j at xlds0 + j*(NT/16)*XPITCH
-
-  // ---- weights: two column fragments of this wave ----
   const int nfr = (N + 31) >> 5;
-  const uint8_t* wptr[NFW];
-  const uint8_t* sptr[NFW];
-#pragma unroll
-  for (int f = 0; f < NFW; ++f) {
-    int F = pid_n * (BN / 32) + nw * NFW + f;
-    F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
-    wptr[f] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 2048 + lane * 16;
-    sptr[f] = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)F * nst * 128 + lr * 4;
+  const int xc = tid & 15;
+  const int xlds0 = (tid >> 4) * XPITCH + xc * 16;  // activation piece j at xlds0 + j*(NT/16)*XPITCH
+  const int grid = (int)gridDim.x;
+  const bool ragged = p.slice_sizes != nullptr;
+  const int nblk = ragged ? p.block_offs[p.n_slices] : 0;
+  const int live = ragged ? nblk * p.grid_n : p.total_tiles;
+  if (ragged) {  // (the host admits at most kMetaSlices slices)
+    for (int i = tid; i < p.n_slices; i += NT) {
+      soffs_s[i] = p.slice_offs[i];
+      ssize_s[i] = p.slice_sizes[i];
+      boffs_s[i] = p.block_offs[i];
+    }
+    if (tid == 0) boffs_s[p.n_slices] = nblk;
   }
+  const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
+
+  // A unit of work = one pass of BM rows over one tile (a row block of one expert x BN columns).  Persistent
+  // workgroups walk over tiles either by a static schedule (round r: tile r * grid + remap(block)) or by claiming them
+  // (TileClaimer); either way the ids of the next two tiles are known when a tile ends, so that a unit's gather
+  // indices and epilogue operands are fetched two and one unit ahead, and its first loads are issued before the
+  // previous unit's epilogue arithmetic.
+  struct Unit {
+    int expert, blk_off, blk_rows, pid_n, start_m, pass_off;
+    bool valid;
+  };
+  auto tile_unit = [&](int pid) __attribute__((always_inline)) -> Unit {
+    Unit u;
+    int eM;
+    if (ragged) {
+      // Tiles are ordered (expert, column tile, row block): the row blocks of one expert that share a column
+      // tile get consecutive ids, run at the same time on one XCD and stream the same weights through its L2.
+      // The expert is the last slice whose first block is not past block pid / grid_n (empty slices share an
+      // offset with their successor): a binary search in the block offsets kept in LDS.
+      const int blk = pid / p.grid_n;
+      int lo = 0, hi = p.n_slices;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (boffs_s[mid] <= blk) lo = mid; else hi = mid;
+      }
+      u.expert = lo;
+      const int first = boffs_s[lo];
+      const int nb = boffs_s[lo + 1] - first;
+      const int local = pid - first * p.grid_n;
+      u.pid_n = local / nb;
+      u.blk_off = (local - u.pid_n * nb) * BLKM;
+      u.start_m = soffs_s[lo];
+      eM = ssize_s[lo];
+    } else {
+      u.pid_n = pid % p.grid_n;
+      u.expert = 0;
+      u.blk_off = (pid / p.grid_n) * BLKM;
+      u.start_m = 0;
+      eM = p.M;
+    }
+    u.blk_rows = (eM - u.blk_off) < BLKM ? (eM - u.blk_off) : BLKM;
+    u.pass_off = 0;
+    u.valid = true;
+    u.expert = __builtin_amdgcn_readfirstlane(u.expert);
+    u.blk_off = __builtin_amdgcn_readfirstlane(u.blk_off);
+    u.blk_rows = __builtin_amdgcn_readfirstlane(u.blk_rows);
+    u.pid_n = __builtin_amdgcn_readfirstlane(u.pid_n);
+    u.start_m = __builtin_amdgcn_readfirstlane(u.start_m);
+    return u;
+  };
+  // the unit after `u`: its next pass, or the first pass of tile `pid_after` (-1: none)
+  auto advance = [&](const Unit& u, int pid_after) __attribute__((always_inline)) -> Unit {
+    Unit n = u;
+    if (u.pass_off + BM < u.blk_rows) {
+      n.pass_off = u.pass_off + BM;
+    } else if (pid_after >= 0) {
+      n = tile_unit(pid_after);
+    } else {
+      n.valid = false;
+    }
+    return n;
+  };
+
+  // (with the same number of tiles for every workgroup the static schedule is already even, and measured faster)
+  const bool dyn = p.tile_counters != nullptr && live % grid != 0;
+  TileClaimer claimer;
+  int round0 = 0;
+  int pid, pid_next;  // this workgroup's current and next tile id (-1 = none)
+  if (dyn) {
+    pid = claimer.init(p.tile_counters, live);
+    pid_next = pid >= 0 ? claimer.second() : -1;
+  } else {
+    const int in0 = live < grid ? live : grid;
+    pid = (int)blockIdx.x < in0 ? xcd_remap(blockIdx.x, in0) : -1;
+    round0 = grid;
+    const int in1 = live - round0 < grid ? live - round0 : grid;
+    pid_next = (pid >= 0 && (int)blockIdx.x < in1) ? round0 + xcd_remap(blockIdx.x, in1) : -1;
+  }
+  int n_tile = 0;  // tiles this workgroup has finished
+  if (ragged) __syncthreads();
+
+  // ---- per-unit operand addresses: a uniform 64-bit base (scalar registers) plus a 32-bit byte offset per lane, so
+  // that they cost one vector register per activation piece and none per weight fragment ----
+  uint32_t xoff[XCH];           // byte offset of this thread's row j in x (x spans less than 4 GiB, checked by the host)
+  const uint8_t* wbase[NFW];    // uniform: first K-stage of this wave's column fragment f
+  const uint8_t* sbase[NFW];
+  const uint32_t lane16 = lane * 16, lr4 = lr * 4;
+  // gather index (source row of x) of tile row `tid` of unit u, rows past the block's end repeat its last row
+  auto unit_gather_index = [&](const Unit& u) __attribute__((always_inline)) -> int {
+    int row = u.blk_off + u.pass_off + tid;
+    row = row < u.blk_off + u.blk_rows ? row : u.blk_off + u.blk_rows - 1;
+    const int srow = u.start_m + row;
+    return p.gather ? p.gather[srow] : srow;
+  };
+  // addresses of unit u from the gather indices staged in gidx_s[set]
+  auto unit_pointers = [&](const Unit& u, int set) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) {
+      const int r = (tid >> 4) + (NT / 16) * j;
+      xoff[j] = (uint32_t)gidx_s[set][r] * (uint32_t)(p.x_stride_m * 2);  // the k offset (incl. this thread's chunk) is added per stage
+    }
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) {
+      int F = u.pid_n * (BN / 32) + nw * NFW + f;
+      F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
+      wbase[f] = p.w + (int64_t)u.expert * p.w_stride_e + (int64_t)F * nst * 2048;
+      sbase[f] = p.w_scale + (int64_t)u.expert * p.ws_stride_e + (int64_t)F * nst * 128;
+    }
+  };
+  // Epilogue operands of a unit as thread `tid` fetches them: bias of tile column tid, gate weight and scatter index of
+  // tile row tid.  `unit_operands` only issues the loads and keeps the raw bits (anything computed from a loaded value
+  // would make the wave wait for it on the spot); `stage_operands` converts them when they go to LDS, a K loop later.
+  uint32_t bias_raw = 0, gam_raw = 0;
+  int dst_raw = 0, gidx_v = 0;
+  auto unit_operands = [&](const Unit& u) __attribute__((always_inline)) {
+    const int off_m = u.blk_off + u.pass_off, blk_end = u.blk_off + u.blk_rows;
+    if (p.bias) {
+      int n = u.pid_n * BN + (tid < BN ? tid : BN - 1);
+      n = n < N ? n : N - 1;
+      const int64_t i = (int64_t)u.expert * p.bias_stride_e + n;
+      bias_raw = p.bias_is_f32 ? static_cast<const uint32_t*>(p.bias)[i] : (uint32_t)static_cast<const uint16_t*>(p.bias)[i];
+    }
+    int row = off_m + (tid < BM ? tid : BM - 1);
+    row = row < blk_end ? row : blk_end - 1;
+    const int srow = u.start_m + row;  // row in expert-sorted order
+    if (p.gammas) gam_raw = p.gammas_is_f32 ? static_cast<const uint32_t*>(p.gammas)[srow] : (uint32_t)static_cast<const uint16_t*>(p.gammas)[srow];
+    if (p.scatter) dst_raw = p.scatter[srow < p.scatter_len ? srow : p.scatter_len - 1];
+  };
+  auto stage_operands = [&](const Unit& u, int set) __attribute__((always_inline)) {
+    // (the index is made opaque so that the LDS addresses are recomputed here instead of being kept in registers)
+    int t = tid;
+    asm volatile("" : "+v"(t));
+    if (t < BN) bias_s[set][t] = p.bias ? bits_f32(p.bias_is_f32 ? bias_raw : bias_raw << 16) : 0.f;
+    if (t < BM) {
+      const int off_m = u.blk_off + u.pass_off, blk_end = u.blk_off + u.blk_rows;
+      const bool ok = off_m + t < blk_end;
+      const int srow = u.start_m + off_m + t;
+      int dst = srow;
+      if (p.scatter) dst = srow < p.scatter_len ? dst_raw : -1;
+      gam_s[set][t] = p.gammas ? bits_f32(p.gammas_is_f32 ? gam_raw : gam_raw << 16) : 1.0f;
+      dst_s[set][t] = ok ? dst : -1;
+      gidx_s[set][t] = gidx_v;
+    }
+  };
 
   typename FR::acc_t acc[NFW][MFW];
-#pragma unroll
-  for (int f = 0; f < NFW; ++f)
-#pragma unroll
-    for (int j = 0; j < MFW; ++j)
-#pragma unroll
-      for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
-
   // activation staging registers, XD stages deep: stage c writes X(c+1) from slot (c+1) % XD to LDS and refills it
   // with X(c+1+XD).  (Native vectors: arrays of the HIP uint4 struct were left in scratch memory here.)
   u32x4_t xreg[XD][XCH];
@@ -745,7 +988,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   auto load_x_piece = [&](int j, int s, int slot) __attribute__((always_inline)) {
     int k0 = s * KC + xc * 8;
     k0 = k0 < K - 8 ? k0 : K - 8;
-    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(xptr[j] + k0 * 2);
+    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(p.x + (xoff[j] + (uint32_t)(k0 * 2)));
   };
   auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
     *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * (NT / 16) * XPITCH) = xreg[slot][j];
@@ -755,9 +998,9 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     s = s < nst ? s : nst - 1;
 #pragma unroll
     for (int f = 0; f < NFW; ++f) {
-      wraw[PAR][f][0] = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 2048);
-      wraw[PAR][f][1] = *reinterpret_cast<const u32x4_t*>(wptr[f] + (int64_t)s * 2048 + 1024);
-      sd[PAR][f] = *reinterpret_cast<const uint32_t*>(sptr[f] + (int64_t)s * 128);
+      wraw[PAR][f][0] = *reinterpret_cast<const u32x4_t*>(wbase[f] + (int64_t)s * 2048 + lane16);
+      wraw[PAR][f][1] = *reinterpret_cast<const u32x4_t*>(wbase[f] + (int64_t)s * 2048 + 1024 + lane16);
+      sd[PAR][f] = *reinterpret_cast<const uint32_t*>(sbase[f] + (int64_t)s * 128 + lr4);
     }
   };
   // operands of step t of the stage held in LDS buffer `buf` / weight registers PAR
@@ -858,18 +1101,25 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     });
   };
 
+  // Stage 0 of a unit (activations of every piece, weights): issued before the previous unit's epilogue arithmetic.
+  auto first_loads = [&]() __attribute__((always_inline)) {
+    static_for<0, XCH>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(S0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int up = 0;             // operand set of the current unit
+  Unit cur_unit;          // the unit being computed
+  int resolve_slot = -1;  // thread 0 writes the claimed tile id into next_tile_s[resolve_slot] before the first barrier
   auto run = [&](auto nj_c, auto gi_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
     constexpr int GI = decltype(gi_c)::value;
     constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
-    // Prologue: stage 0 without overlap.  The order of the loads left in flight (activations, then weights, of
-    // stage 1, then of stage 2) is pinned to the order the steady state leaves them in at the top of a
-    // stage: the compiler's wait counts at the loop header are the merge of both paths, and any mismatch makes
-    // every iteration wait for the loads it has just issued.
-    static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
-    __builtin_amdgcn_sched_barrier(0);
-    load_w(S0, 0);
-    __builtin_amdgcn_sched_barrier(0);
+    // Prologue: finish stage 0 (its loads were issued by first_loads before the previous unit's epilogue).  The order
+    // of the loads left in flight (activations, then weights, of stage 1, then of stage 2) is pinned to the order the
+    // steady state leaves them in at the top of a stage: the compiler's wait counts at the loop header are the merge
+    // of both paths, and any mismatch makes every iteration wait for the loads it has just issued.
     static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, NP>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 1, 1 % XD); });
@@ -886,6 +1136,11 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
       load_w(S2, 2);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // what was fetched during the previous unit's epilogue goes to LDS: this unit's epilogue operands and the next
+    // unit's gather indices (set `up`; its last readers were the epilogue and the address set-up two units back)
+    stage_operands(cur_unit, up);
+    // the claim issued before the previous epilogue has had that long to travel
+    if (resolve_slot >= 0 && tid == 0) next_tile_s[resolve_slot] = claimer.resolve();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -905,9 +1160,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     if (c + 1 < nst) stage(nj_c, gi_c, S1, c + 1);
     if (c + 2 < nst) stage(nj_c, gi_c, S2, c + 2);
   };
-  // row fragments of this wave with valid rows: tile fragments grp, grp + G, ...
-  const int nj = (nfrag_m - grp + G - 1) / G;
-  auto dispatch = [&](auto gi_c) __attribute__((always_inline)) {
+  auto dispatch = [&](auto gi_c, int nj) __attribute__((always_inline)) {
     constexpr int GI = decltype(gi_c)::value;
     if constexpr (GI == 1) {
       if (nj == 0) {
@@ -919,17 +1172,80 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
       if (nj == decltype(n_c)::value) run(n_c, gi_c);
     });
   };
-  if constexpr (G == 2) {
-    if (grp == 1)
-      dispatch(template_int<1>{});
-    else
-      dispatch(template_int<0>{});
-  } else {
-    dispatch(template_int<0>{});
+
+  if (pid >= 0) {
+    Unit& cur = cur_unit;
+    cur = tile_unit(pid);
+    Unit nxt = advance(cur, pid_next);
+    // the first unit has nothing to hide behind: gather indices, addresses, operands, first loads
+    if (tid < BM) gidx_s[1][tid] = unit_gather_index(cur);
+    __syncthreads();
+    unit_pointers(cur, 1);
+    unit_operands(cur);
+    if (nxt.valid && tid < BM) gidx_v = unit_gather_index(nxt);
+    if (dyn && pid_next >= 0) {
+      claimer.issue();  // the tile after the next
+      resolve_slot = 0;
+    }
+    first_loads();
+    for (;;) {
+#pragma unroll
+      for (int f = 0; f < NFW; ++f)
+#pragma unroll
+        for (int j = 0; j < MFW; ++j)
+#pragma unroll
+          for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
+      const int rows = (cur.blk_rows - cur.pass_off) < BM ? (cur.blk_rows - cur.pass_off) : BM;
+      const int nfrag_m = (rows + FM - 1) / FM;  // row fragments that hold valid rows (1..MFW*G)
+      const int nj = (nfrag_m - grp + G - 1) / G;  // those of this wave: tile fragments grp, grp + G, ...
+      if constexpr (G == 2) {
+        if (grp == 1)
+          dispatch(template_int<1>{}, nj);
+        else
+          dispatch(template_int<0>{}, nj);
+      } else {
+        dispatch(template_int<0>{}, nj);
+      }
+      resolve_slot = -1;
+
+      // ---- before this unit's epilogue: everything the next units need from memory ----
+      const int ncol0 = cur.pid_n * BN + nw * NFW * FM;
+      Unit nxt2 = nxt;
+      if (nxt.valid) {
+        if (cur.pass_off + BM >= cur.blk_rows) {
+          // the next unit opens a new tile; the tile after it was claimed during this tile's first prologue (or
+          // follows statically)
+          pid = pid_next;
+          ++n_tile;
+          if (dyn) {
+            pid_next = __builtin_amdgcn_readfirstlane(next_tile_s[(n_tile - 1) & 1]);
+          } else {
+            round0 += grid;
+            const int in_round = live - round0 < grid ? live - round0 : grid;
+            pid_next = (int)blockIdx.x < in_round ? round0 + xcd_remap(blockIdx.x, in_round) : -1;
+          }
+          if (dyn && pid_next >= 0) {
+            claimer.issue();
+            resolve_slot = n_tile & 1;
+          }
+        }
+        nxt2 = advance(nxt, pid_next);
+        // (these loads and the claim come BEFORE the next unit's first loads: the number of them in flight differs
+        // from path to path, and only what is issued after a load makes the wait for that load inexact)
+        unit_operands(nxt);
+        if (nxt2.valid && tid < BM) gidx_v = unit_gather_index(nxt2);
+        __builtin_amdgcn_sched_barrier(0);
+        unit_pointers(nxt, up);
+        first_loads();
+      }
+      staged_epilogue<G, MFW, NFW, SWIGLU>(p, acc, yrsrc, bias_s[up], gam_s[up], dst_s[up], nw * NFW * FM, ncol0, grp, lr, h);
+      if (!nxt.valid) break;
+      cur = nxt;
+      nxt = nxt2;
+      up ^= 1;
+    }
   }
-  gemm_epilogue<FM, G, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, blk_off + blk_rows, pid_n * BN + nw * NFW * FM, pid_n * BN + BN <= N, grp, lr, h);
-  }  // passes
-  }  // rounds
+  if (dyn) claimer.finish();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1146,10 +1462,21 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   const int K = p.K, N = p.N;
   const int nst = p.w_nst;  // stages of 256 (two 4 KiB weight blocks per column fragment each)
   const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
-  for (int round0 = 0; round0 < live; round0 += (int)gridDim.x) {
-  const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
-  if ((int)blockIdx.x >= in_round) break;
-  const int pid = round0 + xcd_remap(blockIdx.x, in_round);
+  __shared__ int next_tile_s[2];  // written by thread 0 before a tile's first barrier: the id of the tile after it
+  int tile_par = 0, n_tile = 0;
+  const bool dyn = p.tile_counters != nullptr;
+  TileClaimer claimer;
+  int pid = claimer.init(p.tile_counters, live), round0 = 0;
+  // (dynamic: a workgroup whose queue is shorter than its first index gets no tile at all, which only happens when
+  // there are fewer tiles than workgroups; its first two tiles are fixed, later ones are claimed)
+  const int pid_second = claimer.second();
+  if (!dyn) {
+    const int in_round0 = live < (int)gridDim.x ? live : (int)gridDim.x;
+    pid = (int)blockIdx.x < in_round0 ? xcd_remap(blockIdx.x, in_round0) : -1;
+  }
+  while (pid >= 0) {
+  const bool claim_now = dyn && (n_tile >= 1 || pid_second < 0);
+  if (claim_now) claimer.issue();  // the next tile's claim travels while this tile's first loads do
   int expert, blk_off, start_m, eM, pid_n;
   if (p.slice_sizes) {
     expert = p.block_sched[pid / p.grid_n] & 0xFFFF;
@@ -1301,6 +1628,8 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, NFW * NS>([&](auto wc) __attribute__((always_inline)) { load_w(S1, decltype(wc)::value % NFW, decltype(wc)::value / NFW, 1); });
     __builtin_amdgcn_sched_barrier(0);
+    // the claim issued when the tile started has had the prologue's loads to travel behind
+    if (claim_now && pass_off == 0 && tid == 0) next_tile_s[tile_par ^ 1] = claimer.resolve();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -1321,7 +1650,20 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   gemm_epilogue<FM, 1, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, blk_off + blk_rows, pid_n * BN + nw * NFW * FM,
                                          pid_n * BN + BN <= N, 0, lr, h);
   }  // passes
-  }  // rounds
+  // next tile
+  if (dyn) {
+    // written by thread 0 before this tile's first workgroup barrier; the slot is not written again before the
+    // first barrier of the tile after the next, which no wave passes before it has read this value
+    tile_par ^= 1;
+    pid = claim_now ? __builtin_amdgcn_readfirstlane(next_tile_s[tile_par]) : pid_second;
+    ++n_tile;
+  } else {
+    round0 += (int)gridDim.x;
+    const int in_round = live - round0 < (int)gridDim.x ? live - round0 : (int)gridDim.x;
+    pid = (int)blockIdx.x < in_round ? round0 + xcd_remap(blockIdx.x, in_round) : -1;
+  }
+  }  // tiles
+  if (dyn) claimer.finish();
 }
 
 template <int MR>
@@ -1390,9 +1732,8 @@ int32_t launch_mxn(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   q.total_tiles = (int32_t)grid;
-  // persistent grid: as many workgroups as fit on the device at once (LDS decides how many share a CU)
-  const int per_cu = LDS_BYTES > 80 * 1024 ? 1 : 2;
-  const int64_t resident = (int64_t)busy_cu_count(p.idle_cus) * per_cu;
+  // persistent grid: one workgroup per CU (a wave's registers leave no room for a second one on its SIMD)
+  const int64_t resident = (int64_t)busy_cu_count(p.idle_cus);
   if (grid > resident) grid = resident;
   auto launch = [&](auto kern) -> int32_t {
     if (const int32_t rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES)) return rc;
@@ -1543,6 +1884,8 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.bias_vec = d->bias && (d->bias_stride_e % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->bias) & 15) == 0);
   p.grid_n = 0;
   p.idle_cus = d->idle_cus;
+  p.tile_counters = d->tile_counters;
+  p.y_bytes = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
   if (d->w_layout == TK_W_TILED && d->w_dtype == TK_E4M3) {
@@ -1561,6 +1904,26 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
     if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);
+    if (d->block_m >= 64) {
+      // the prefill kernels address activation rows with 32-bit byte offsets from x
+      const int64_t rows = d->x_rows > 0 ? d->x_rows : (d->gather_indx ? 0 : d->M);
+      if (d->x_stride_m * 2 >= (int64_t)1 << 32 || rows * d->x_stride_m * 2 > (int64_t)1 << 32)
+        return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations of 4 GiB and more are not supported with tiled MXFP4 weights (%lld rows, row stride %lld)", (long long)rows, (long long)d->x_stride_m);
+    }
+    if (d->block_m >= 64) {
+      // the prefill kernels store through a buffer resource with 16-byte (8-byte with swiglu) pieces per lane: rows
+      // must be 16-byte aligned and long enough to take the last piece whole
+      const int64_t n_out = swiglu ? d->N / 2 : d->N;
+      const int64_t piece = swiglu ? 4 : 8;
+      const int64_t y_rows = d->scatter_indx ? d->scatter_len : d->M;
+      const int64_t y_bytes = y_rows * d->y_stride_m * 2;
+      if (!p.y_vec || d->y_stride_m < cdiv(n_out, piece) * piece)
+        return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: with tiled MXFP4 weights at block_m >= 64 output rows must be 16-byte aligned and padded to a multiple of %lld columns (row stride %lld for %lld columns)", (long long)piece, (long long)d->y_stride_m, (long long)n_out);
+      if (y_bytes >= (int64_t)1 << 31) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: outputs of 2 GiB and more are not supported with tiled MXFP4 weights");
+      p.y_bytes = (uint32_t)y_bytes;
+    }
+    if (d->block_m >= 64 && d->n_slices > kMetaSlices) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: at most %d slices with tiled MXFP4 weights at block_m >= 64 (got %d)", kMetaSlices, d->n_slices);
+    if (d->block_m >= 64 && (d->x_row_scale || d->w_col_scale)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: per-row / per-column scales are not supported with tiled MXFP4 weights at block_m >= 64");
     if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w_mx_scale) & 3) || d->ws_stride_e % 4) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
     const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");

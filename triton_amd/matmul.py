@@ -102,6 +102,24 @@ def matmul_set_idle_sms(num_idle_sms):
     set_idle_sms(num_idle_sms)
 
 
+_TILE_COUNTERS: dict = {}
+_STATIC_TILES = False  # True: the persistent kernels walk their static tile schedule (for comparisons)
+
+
+def _tile_counters(device: torch.device) -> torch.Tensor:
+    """Zeroed int32 words the persistent kernels claim tiles with (`tk_gemm_desc.tile_counters`): one small buffer
+    per (device, stream), made on first use and kept for the life of the process.  A kernel leaves the words zero, so
+    launches in stream order share them; launches on different streams get different buffers.  (A buffer first made
+    while a HIP graph is being captured belongs to the capture stream: graphs captured on one stream must not be
+    replayed concurrently with each other.)"""
+    key = (device.index, nt.stream_ptr(device))
+    buf = _TILE_COUNTERS.get(key)
+    if buf is None:
+        buf = torch.zeros(16, dtype=torch.int32, device=device)
+        _TILE_COUNTERS[key] = buf
+    return buf
+
+
 def _flex_out_is_trivial(flex: FlexCtx) -> bool:
     return (flex.acc_data.scale is None and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
             and flex.out_data.checksum_scale is None)
@@ -307,6 +325,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.x = a.data_ptr()
     d.x_dtype = nt.TORCH_TO_TK[a.dtype]
     d.x_stride_m = a.stride(0)
+    d.x_rows = a.shape[0]
     a_ts = precision_config.a_mx_tensor_scale
     if a_ts is not None:
         a_ts = a_ts.to(torch.float32).reshape(-1).contiguous()
@@ -420,13 +439,24 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         d.grid_m = (M + block_m - 1) // block_m
     d.block_m = block_m
     d.M, d.N, d.K = M, N, K
-    d.y = c.data_ptr()
+    y_buf = c
+    if tiled and block_m >= 64:
+        # the prefill kernels write whole 16-byte pieces through a buffer resource: rows 16-byte aligned and padded to
+        # a multiple of 8 columns; an output that is not goes through a padded buffer and is copied
+        n_pad = (out_shape[1] + 7) // 8 * 8
+        if c.stride(0) % 8 or c.data_ptr() % 16 or c.stride(0) < n_pad:
+            y_buf = torch.empty((out_shape[0], n_pad), dtype=c.dtype, device=c.device)[:, :out_shape[1]]
+    d.y = y_buf.data_ptr()
     d.y_dtype = nt.TORCH_TO_TK[c.dtype]
-    d.y_stride_m = c.stride(0)
+    d.y_stride_m = y_buf.stride(0)
     d.activation = act
     d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
     d.idle_cus = max(0, int(opt_flags.idle_sms or 0))
+    if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES:
+        d.tile_counters = _tile_counters(a.device).data_ptr()
     with nt.on_device(a.device):
         nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
     del keep
+    if y_buf is not c:
+        c.copy_(y_buf)
     return c
