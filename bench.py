@@ -276,6 +276,45 @@ def bench_fp8(device, steps, warmup):
                 frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4))
 
 
+def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
+    """Config 3's shapes on the scaled-MFMA path: the activations are MX-quantised (e4m3 + one e8m0 scale per 32 along
+    K) and multiplied with the MXFP4 weights by v_mfma_scale_f32_32x32x64_f8f6f4, both operands in their storage
+    formats; the first GEMM's epilogue quantises its fp32 accumulator to MXFP8 for the second.  Not the headline:
+    config 3 states bf16 activations, and this path is checked against an oracle fed the same quantised activations.
+    One step = router, quantise x, GEMM1 (+bias, swiglu, MX output), GEMM2 (+bias, gate weight), combine."""
+    from triton_kernels.legacy import routing
+    from triton_kernels.matmul import Epilogue, FnName, FnSpecs, FusedActivation, PrecisionConfig, matmul
+    from triton_kernels.numerics_details.mxfp import downcast_to_mxfp, quantize_mxfp8_fn
+    from triton_kernels.reduce import reduce
+    from triton_kernels.swiglu import swiglu_fn
+    T, d = x.shape
+    W = weights
+    f2 = W["b1"].shape[-1]
+    act = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0))
+    epi = Epilogue(FnSpecs(FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn, (), ()), tuple(), tuple(), effective_itemsize=1.0)
+    h_scale = torch.empty((T * k, (f2 // 2) // 32), dtype=torch.uint8, device=device)
+
+    def step():
+        rdata, _, scatter = routing(logits, k)
+        xq, xs = downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
+        h = matmul(xq, W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, fused_activation=act, epilogue=epi,
+                   precision_config=PrecisionConfig(a_mx_scale=xs, b_mx_scale=W["w1s"], c_mx_scale=h_scale, out_dtype=torch.float8_e4m3fn))
+        y = matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=scatter.dst_indx, gammas=rdata.gate_scal,
+                   precision_config=PrecisionConfig(a_mx_scale=h_scale, b_mx_scale=W["w2s"], out_dtype=torch.bfloat16))
+        return reduce(y.view(T, k, -1), dim=1)[0]
+
+    ms = time_steps(step, steps, warmup)
+    flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
+    # algorithmic bytes with one-byte activations: x_q + scales, W1, h_q twice, W2, y twice, out (SURVEY accounting)
+    R = T * k
+    E = W["b1"].shape[0]
+    nbytes = (R * d * 33 / 32 + E * (d * f2 * 17 / 32 + f2 * 2) + 2 * R * (f2 // 2) * 33 / 32 + E * ((f2 // 2) * d * 17 / 32 + d * 2) + 2 * R * d * 2 + T * d * 2)
+    t_roof_ms = max(flops / 5.0e15, nbytes / (PEAK_HBM_GBPS * 1e9)) * 1e3
+    return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8 (MXFP8 x MXFP4, scaled MFMA)",
+                frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), t_roof_ms=round(t_roof_ms, 4), frac=round(t_roof_ms / ms, 4),
+                bound="hbm" if nbytes / (PEAK_HBM_GBPS * 1e9) > flops / 5.0e15 else "mfma")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -371,7 +410,8 @@ def main():
     rec["layer_roofline"] = {"t_roof_ms": round(t_roof_ms, 4), "frac": round(t_roof_ms / ms, 4),
                              "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1)}
     if not args.no_extra:
-        rec["extra"] = {"fp8_config5": bench_fp8(device, max(5, args.steps // 2), 2),
+        rec["extra"] = {"scaled_mfma_config3": bench_scaled_mfma(device, weights, x, logits, k, args.steps, args.warmup),
+                        "fp8_config5": bench_fp8(device, max(5, args.steps // 2), 2),
                         "decode_config4": bench_decode(device, max(5, args.steps), args.warmup),
                         "mx_round_trip_config2": bench_mx(device, max(5, args.steps), args.warmup)}
     if not args.no_cpu:

@@ -247,7 +247,7 @@ enum tk_activation {
 typedef struct tk_gemm_desc {
   /* activations: [rows, K], unit stride along K */
   const void* x;
-  int32_t x_dtype; /* TK_BF16, or TK_E4M3 with x_row_scale */
+  int32_t x_dtype; /* TK_BF16, TK_E4M3 with x_row_scale (plain fp8), or TK_E4M3 with x_mx_scale (MXFP8) */
   int64_t x_stride_m;
   const float* x_row_scale; /* fp32 per row of x, read at the source row src(r), or NULL */
   /* weights: [E, K, N]; e2m1 is packed two per byte along K and the strides count bytes */
@@ -279,7 +279,7 @@ typedef struct tk_gemm_desc {
   int32_t M, N, K; /* M: rows of the single slice when not ragged; N: columns of W; K: reduction */
   /* output [rows, N or N/2], unit stride along N */
   void* y;
-  int32_t y_dtype; /* TK_BF16 */
+  int32_t y_dtype; /* TK_BF16, or TK_E4M3 with y_mx_scale */
   int64_t y_stride_m;
   int32_t activation; /* enum tk_activation */
   float act_alpha, act_limit;
@@ -298,6 +298,18 @@ typedef struct tk_gemm_desc {
   /* rows of x (with gather_indx: every index is below it); 0 = not stated (then M when not gathering).  The kernels
    * for tiled MXFP4 weights at block_m >= 64 need x to span less than 4 GiB and refuse larger ones. */
   int64_t x_rows;
+  /* MXFP8 activations (x_dtype TK_E4M3): e8m0 block scales uint8 [rows of x, K / 32], unit stride along K, one per
+   * 32 consecutive k of a row (tk/matmul.py:130-132 `a_mx_scale`); NULL = x is not MX-quantised.  Goes with tiled
+   * MXFP4 weights, block_m 128 or 256, and runs on v_mfma_scale_f32_32x32x64_f8f6f4 with both operands in their
+   * storage formats. */
+  const void* x_mx_scale;
+  int64_t xs_stride_m;
+  /* MX-quantised output (y_dtype TK_E4M3, MXFP8-activation path only): the epilogue quantises the fp32 accumulator,
+   * after bias, activation and gate weight, in blocks of 32 output columns (the `QUANTIZE_MXFP8` epilogue,
+   * tk/matmul_details/_matmul.py:593-637): e4m3 bytes to y, one e8m0 byte per block to y_mx_scale
+   * [rows of y, N_out / 32].  NULL = plain bf16 output. */
+  void* y_mx_scale;
+  int64_t ys_stride_m;
 } tk_gemm_desc;
 
 #define TK_GEMM_TILE_COUNTER_WORDS 16

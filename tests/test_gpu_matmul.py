@@ -387,3 +387,96 @@ def test_standalone_swiglu_with_routing_data(mods, device):
     ref = omoe.swiglu(a, 1.702, 7.0)
     assert int(rdata.expt_data.slice_offs[E]) == 50
     assert_close(ref[:50], out[:50], what="swiglu rows")
+
+
+def _mx_activations(x):
+    """MXFP8 (e4m3 + e8m0 per 32 along K) quantisation of x with the oracle, and what it dequantises to."""
+    xq, xs = omx.downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
+    return xq, xs, omx.upcast_from_mxfp(xq, xs, torch.bfloat16, axis=-1)
+
+
+@pytest.mark.parametrize("m, n, k", [(16, 256, 256), (300, 400, 416), (1000, 704, 800), (256, 1024, 512), (1500, 512, 1024)])
+@pytest.mark.parametrize("block_m", [128, 256])
+@pytest.mark.parametrize("do_gather, do_scatter, do_gamma, swiglu", [(False, False, False, False), (True, False, False, True),
+                                                                      (False, True, True, False), (True, True, True, False)])
+def test_matmul_mxfp8_activations(mods, device, m, n, k, block_m, do_gather, do_scatter, do_gamma, swiglu):
+    """MXFP8 activations x MXFP4 weights (`PrecisionConfig.a_mx_scale`; the reference's cases:
+    tests/test_matmul.py:207-216) on the scaled MFMA.  The oracle is fed the SAME quantised activations, dequantised
+    to bf16 as the reference's `apply_precision` does (matmul.py:783-795): both operands are then exact in bf16 and only
+    the accumulation order differs, so the bf16 GEMM tolerance applies."""
+    mm, sw_mod, tensor = mods
+    g = torch.Generator().manual_seed(m * 5 + n + k + block_m)
+    n_slices = 10
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    xq, xs, x_deq = _mx_activations(x)
+    W = _make_w(n_slices, k, n, "mxfp4_tiled", g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    gi = torch.randint(0, m, (m, ), generator=g, dtype=torch.int32) if do_gather else None
+    sc = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    if sc is not None and m > 20:
+        sc[torch.rand(m, generator=g) < 0.05] = -1
+    gam = 2.0**torch.randint(-5, 0, (m, ), generator=g).float() if do_gamma else None
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw_mod.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    pc = mm.PrecisionConfig(a_mx_scale=xs.to(device), b_mx_scale=W["scale_dev"], out_dtype=torch.bfloat16)
+    dv = lambda t: None if t is None else t.to(device)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(xq.to(device), W["w_dev"], bias.to(device), md, gather_indx=dv(gi), scatter_indx=dv(sc), gammas=dv(gam),
+                      precision_config=pc, fused_activation=act)
+    ref = omoe.matmul(x_deq, W["w_cpu"], bias, sizes, gather_indx=gi, scatter_indx=sc, gammas=gam, w_mx_scale=W["scale_cpu"],
+                      out_dtype=torch.float32 if swiglu else torch.bfloat16)
+    if swiglu:
+        ref = omoe.swiglu(ref, 1.702, 7.0).to(torch.bfloat16)
+    got = y.cpu()
+    if sc is not None:  # rows that no entry writes are undefined in the kernel path, zero in the oracle
+        written = torch.zeros(m, dtype=torch.bool)
+        written[sc[sc >= 0].long()] = True
+        got = torch.where(written[:, None], got, torch.zeros_like(got))
+    assert y.dtype == torch.bfloat16 and got.shape == ref.shape
+    assert_close(ref, got, maxtol=3e-2, what="y")
+    assert_allclose_gate(ref, got, what="y")
+
+
+@pytest.mark.parametrize("swiglu, scatter", [(True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("block_m", [128, 256])
+def test_mxfp8_activations_with_fused_mx_output(mods, device, swiglu, scatter, block_m):
+    """With MXFP8 activations the `QUANTIZE_MXFP8` epilogue runs inside the GEMM, on the fp32 accumulator
+    (matmul_details/_matmul.py:593-637).  Against the oracle's GEMM (fp32 result) -> MX quantisation: (1) block scales
+    equal except where the two fp32 sums put a block's maximum on different sides of a power-of-two boundary (a handful
+    of blocks at most), (2) dequantised values within the reference's tolerance for this epilogue (maxtol 4e-1 /
+    rmstol 4e-2, tests/test_matmul.py:627-643), (3) nearly all codes bit-equal."""
+    mm, sw_mod, tensor = mods
+    from triton_amd.numerics_details.mxfp import quantize_mxfp8_fn
+    g = torch.Generator().manual_seed(23 + block_m)
+    m, n, k, n_slices = 600, 512, 416, 6
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    xq, xs, x_deq = _mx_activations(x)
+    W = _make_w(n_slices, k, n, "mxfp4_tiled", g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    sc = torch.randperm(m, generator=g).to(torch.int32) if scatter else None
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw_mod.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    n_out = n // 2 if swiglu else n
+    epi = mm.Epilogue(mm.FnSpecs(mm.FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn, (), ()), tuple(), tuple(), effective_itemsize=6.0)
+    c_scale = torch.full((m, n_out // 32), 0xFF, dtype=torch.uint8, device=device)
+    pc = mm.PrecisionConfig(a_mx_scale=xs.to(device), b_mx_scale=W["scale_dev"], c_mx_scale=c_scale, out_dtype=torch.float8_e4m3fn)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        yq = mm.matmul(xq.to(device), W["w_dev"], bias.to(device), md, precision_config=pc, epilogue=epi, fused_activation=act,
+                       scatter_indx=None if sc is None else sc.to(device))
+    assert yq.dtype == torch.float8_e4m3fn and yq.shape == (m, n_out) and pc.c_mx_scale is c_scale
+    h = omoe.matmul(x_deq, W["w_cpu"], bias, sizes, w_mx_scale=W["scale_cpu"], scatter_indx=sc, out_dtype=torch.float32)
+    if swiglu:
+        h = omoe.swiglu(h, 1.702, 7.0)
+    q_ref, s_ref = omx.downcast_to_mxfp(h, torch.float8_e4m3fn, axis=-1)
+    s_got, q_got = c_scale.cpu(), yq.cpu()
+    scale_diff = (s_ref != s_got).float().mean().item()
+    assert scale_diff <= 2e-3, f"{scale_diff:.4g} of the block scales differ from the oracle's"
+    code_diff = (q_ref.view(torch.uint8) != q_got.view(torch.uint8)).float().mean().item()
+    assert code_diff <= 0.02, f"{code_diff:.4g} of the e4m3 codes differ from the oracle's"
+    ref = omx.upcast_from_mxfp(q_ref, s_ref, torch.bfloat16, axis=-1)
+    got = omx.upcast_from_mxfp(q_got, s_got, torch.bfloat16, axis=-1)
+    assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
+    # the quantised result is close to the unquantised GEMM (e4m3 has 3 mantissa bits: half a step is 2^-4 relative)
+    assert_close(h, got, maxtol=1.0, rmstol=4e-2, what="MX output against the unquantised result")

@@ -64,6 +64,7 @@ class GemmDesc(_c.Structure):
         ("y", _ptr), ("y_dtype", _i32), ("y_stride_m", _i64),
         ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
         ("w_layout", _i32), ("idle_cus", _i32), ("tile_counters", _ptr), ("x_rows", _i64),
+        ("x_mx_scale", _ptr), ("xs_stride_m", _i64), ("y_mx_scale", _ptr), ("ys_stride_m", _i64),
     ]
 
 

@@ -233,16 +233,36 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         fused_activation = FusedActivation(FnSpecs.default(), tuple())
     if epilogue is None:
         epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+    # MXFP8 activations (`a_mx_scale`): e4m3 values with one e8m0 scale per 32 k, multiplied with tiled MXFP4 weights
+    # on the scaled MFMA (triton_kernels/matmul.py:130-132,783-795)
+    a_scale = precision_config.a_mx_scale
+    mx_act = a_scale is not None
+    if mx_act:
+        if isinstance(a_scale, Tensor):
+            if not isinstance(a_scale.storage.layout, StridedLayout):
+                raise NotImplementedError(f"activation scale layout {type(a_scale.storage.layout).__name__} is not supported")
+            a_scale = a_scale.storage.data
+        if not (isinstance(b, Tensor) and isinstance(b.storage.layout, GFX950MXValueLayout)):
+            raise NotImplementedError("MX-quantised activations (a_mx_scale) need MXFP4 weights in the tiled layout "
+                                      "(convert them with make_default_matmul_mxfp4_w_layout)")
+        assert a_scale.dtype == torch.uint8, f"Unsupported microscale dtype {a_scale.dtype}"
+        assert precision_config.a_microblock_size in (None, MXFP_BLOCK_SIZE), \
+            f"Unsupported microscale block size {precision_config.a_microblock_size}"
+    mx_out_fused = False
     if epilogue.specs.name in (FnName.QUANTIZE_MXFP8.name, FnName.QUANTIZE_MXFP4.name):
-        return _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
-                              fused_activation, epilogue)
-    if epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
+        # with MXFP8 activations the kernel quantises its fp32 accumulator itself; otherwise the bf16 GEMM is followed
+        # by the MX quantiser
+        mx_out_fused = (mx_act and epilogue.specs.name == FnName.QUANTIZE_MXFP8.name
+                        and precision_config.out_dtype == torch.float8_e4m3fn and precision_config.c_mx_scale is not None
+                        and precision_config.c_microblock_size in (None, MXFP_BLOCK_SIZE))
+        if not mx_out_fused:
+            return _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
+                                  fused_activation, epilogue)
+    elif epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
         raise NotImplementedError(f"epilogue {epilogue.specs.name!r} is not supported (MXFP8 / MXFP4 output quantisation only)")
     flex = precision_config.flex_ctx
     if not _flex_out_is_trivial(flex):
         raise NotImplementedError("flexpoint output / accumulator scales are not supported (outputs are bf16)")
-    if precision_config.a_mx_scale is not None:
-        raise NotImplementedError("MX-quantised activations (a_mx_scale) are not supported")
     if isinstance(a, Tensor):
         a = a.storage.data
     a = flex.lhs_data.reinterpret(a)
@@ -306,10 +326,23 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         has_limit = int(lim is not None)
         limit = float(lim) if lim is not None else 0.0
     out_dtype = precision_config.out_dtype or a.dtype
-    if out_dtype != torch.bfloat16:
+    if out_dtype != torch.bfloat16 and not mx_out_fused:
         raise NotImplementedError(f"output dtype {out_dtype} is not supported (bf16 only); set precision_config.out_dtype")
     y_rows = scatter_indx.shape[0] if scatter_indx is not None else M
     out_shape = (y_rows, N // reduction_n)
+    c_scale = None
+    if mx_out_fused:
+        c_scale = precision_config.c_mx_scale
+        if isinstance(c_scale, Tensor):
+            if not isinstance(c_scale.storage.layout, StridedLayout):
+                raise NotImplementedError(f"output scale layout {type(c_scale.storage.layout).__name__} is not supported")
+            c_scale = c_scale.storage.data
+        if out_shape[1] % MXFP_BLOCK_SIZE != 0:
+            raise NotImplementedError(f"MX-quantised output needs N_out % 32 == 0 (got {out_shape[1]})")
+        assert c_scale.dtype == torch.uint8 and tuple(c_scale.shape[-2:]) == (y_rows, out_shape[1] // MXFP_BLOCK_SIZE) \
+            and c_scale.stride(-1) == 1, f"c_mx_scale must be uint8 [{y_rows}, {out_shape[1] // MXFP_BLOCK_SIZE}]"
+        precision_config.c_microblock_size = MXFP_BLOCK_SIZE
+        precision_config.c_value_pack_factor = 1
     if c is None:
         c = torch.empty(out_shape, dtype=out_dtype, device=a.device)
     else:
@@ -340,6 +373,18 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if a_ts is not None:
         d.x_row_scale = a_ts.data_ptr()
     keep = [a_ts]
+    if mx_act:
+        if a.dtype != torch.float8_e4m3fn:
+            raise NotImplementedError(f"MX-quantised activations must be float8_e4m3fn (got {a.dtype})")
+        if a_ts is not None:
+            raise NotImplementedError("a_mx_tensor_scale / flexpoint scales are not supported with a_mx_scale")
+        assert tuple(a_scale.shape) == (a.shape[0], (K + MXFP_BLOCK_SIZE - 1) // MXFP_BLOCK_SIZE), \
+            f"a_mx_scale must be [{a.shape[0]}, {(K + 31) // 32}], got {tuple(a_scale.shape)}"
+        if a_scale.stride(-1) != 1:
+            a_scale = a_scale.contiguous()
+        d.x_mx_scale = a_scale.data_ptr()
+        d.xs_stride_m = a_scale.stride(0)
+        keep.append(a_scale)
     if tiled_fp8:
         if b_scale is not None:
             raise NotImplementedError("MX scales are supported with mxfp4 (uint8) weights only")
@@ -418,6 +463,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     block_m = opt_flags.block_m
     if tiled_fp8:
         block_m = 256 if block_m == 256 else 128  # the FP8 MFMA kernel's row blocks
+    elif mx_act:
+        from .matmul_details.opt_flags import _get_opt_flags_constraints
+        forced = _get_opt_flags_constraints().get("block_m")
+        block_m = 256 if (forced == 256 or (forced is None and is_ragged and M <= 144 * n_slices)) else 128
     elif tiled:
         from .matmul_details.opt_flags import _get_opt_flags_constraints
         if block_m == 128 and _get_opt_flags_constraints().get("block_m") is None and is_ragged and M <= 144 * n_slices:
@@ -440,7 +489,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.block_m = block_m
     d.M, d.N, d.K = M, N, K
     y_buf = c
-    if tiled and block_m >= 64:
+    if tiled and block_m >= 64 and not mx_act:
         # the prefill kernels write whole 16-byte pieces through a buffer resource: rows 16-byte aligned and padded to
         # a multiple of 8 columns; an output that is not goes through a padded buffer and is copied
         n_pad = (out_shape[1] + 7) // 8 * 8
@@ -452,7 +501,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.activation = act
     d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
     d.idle_cus = max(0, int(opt_flags.idle_sms or 0))
-    if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES:
+    if c_scale is not None:
+        d.y_mx_scale = c_scale.data_ptr()
+        d.ys_stride_m = c_scale.stride(-2)
+    if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES and not mx_act:
         d.tile_counters = _tile_counters(a.device).data_ptr()
     with nt.on_device(a.device):
         nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
