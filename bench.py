@@ -74,11 +74,11 @@ class MoeLayer:
     """The hot path composed from the drop-in API (triton_kernels names)."""
 
     def __init__(self, weights, k, alpha=1.702, limit=7.0):
-        from triton_kernels.legacy import routing
+        from triton_kernels.legacy import matmul_ogs, routing
         from triton_kernels.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
         from triton_kernels.reduce import reduce
         from triton_kernels.swiglu import swiglu_fn
-        self.routing, self.matmul, self.reduce = routing, matmul, reduce
+        self.routing, self.matmul, self.reduce, self.matmul_ogs = routing, matmul, reduce, matmul_ogs
         self.W = weights
         self.k = k
         self.act = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (alpha, limit))
@@ -97,9 +97,8 @@ class MoeLayer:
         md = rdata.expt_data
         h = self.matmul(x, W["w1"], W["b1"], md, gather_indx=rdata.token_indx, precision_config=self.pc1,
                         fused_activation=self.act)
-        y = self.matmul(h, W["w2"], W["b2"], md, scatter_indx=scatter.dst_indx, precision_config=self.pc2,
-                        gammas=rdata.gate_scal)
-        out, _ = self.reduce(y.view(x.shape[0], k, -1), dim=1)
+        # scatter-GEMM and top-k combine through the legacy entry point: one launch at decode shapes, GEMM + reduce otherwise
+        out = self.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=self.pc2, gammas=rdata.gate_scal)
         return out, rdata
 
 
@@ -171,10 +170,10 @@ def capture(fn):
 
 
 def bench_decode(device, steps, warmup):
-    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched.  The whole
-    layer (router, two GEMMs, combine: 6 launches) is replayed from a HIP graph, as a serving loop would; three
-    weight copies are rotated so no step finds its weights in the last-level cache.  Every replay's output is
-    checked against the eager result before timing."""
+    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched.  Three layers with
+    their own weight copies (so that no layer finds its weights in the last-level cache) are captured in ONE HIP graph,
+    as a serving loop captures a decode step over all its layers; the time of a layer is the replay time / 3.  Every
+    layer's output of every checked replay is compared with the eager result before timing."""
     E, k, d, f2 = 128, 4, 2880, 5760
     copies = [to_matmul_layout(w) for w in make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)]
     per_expert = d * f2 // 2 + d * f2 // 32 + (f2 // 2) * d // 2 + (f2 // 2) * d // 32
@@ -182,36 +181,31 @@ def bench_decode(device, steps, warmup):
     g = torch.Generator().manual_seed(3)
     ebias = torch.randn((E, ), generator=g) * 1.5
     layers = [MoeLayer(w, k) for w in copies]
+    n_layers = len(layers)
     for T in (1, 4, 16, 64):
         x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
         logits = (torch.randn((T, E), generator=g) + ebias).to(device)
         eager = [layer(x, logits) for layer in layers]
         active = int((eager[0][1].expt_hist > 0).sum())
-        it = [0]
 
         def step_eager():
-            layers[it[0] % len(layers)](x, logits)
-            it[0] += 1
+            for layer in layers:
+                layer(x, logits)
 
-        ms_eager = time_steps(step_eager, steps, warmup)
-        graphs = [capture(lambda layer=layer: layer(x, logits)[0]) for layer in layers]
-        for rep in range(2):  # replays with eager work in between, each compared with the eager output
-            for (gr, out), (ref, _) in zip(graphs, eager):
-                gr.replay()
-                torch.cuda.synchronize()
+        ms_eager = time_steps(step_eager, steps, warmup) / n_layers
+        graph, outs = capture(lambda: [layer(x, logits)[0] for layer in layers])
+        for rep in range(2):  # replays with eager work in between, each compared with the eager outputs
+            graph.replay()
+            torch.cuda.synchronize()
+            for out, (ref, _) in zip(outs, eager):
                 if not torch.equal(out, ref):
                     raise RuntimeError(f"decode T={T}: graph replay {rep} differs from the eager result")
             step_eager()
-
-        def step_graph():
-            graphs[it[0] % len(graphs)][0].replay()
-            it[0] += 1
-
-        ms = time_steps(step_graph, steps, warmup)
+        ms = time_steps(graph.replay, steps, warmup) / n_layers
         gbytes = active * per_expert / 1e9
         res[f"T{T}"] = dict(ms=round(ms, 4), ms_eager=round(ms_eager, 4), active_experts=active, weight_GB=round(gbytes, 4),
                             GBps=round(gbytes / (ms * 1e-3), 1), frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
-        del graphs
+        del graph
     return res
 
 

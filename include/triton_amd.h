@@ -310,12 +310,52 @@ typedef struct tk_gemm_desc {
    * [rows of y, N_out / 32].  NULL = plain bf16 output. */
   void* y_mx_scale;
   int64_t ys_stride_m;
+  /* Fused top-k combine behind the scatter (decode: tiled MXFP4 weights, block_m 16 or 32, no activation):
+   * scatter_indx maps expert-sorted row r to flat position t * combine_k + j; besides y [tokens * combine_k, N] the
+   * kernel writes combine_out[t, :] = sum over j of y[t * combine_k + j, :] (fp32 sum in j order, bf16 result: what
+   * tk_reduce_mid computes from y), by the wave that completes token t's rows last.  combine_counters:
+   * tokens * ceil(N / 32) zeroed int32 words, left zero.  A token with fewer than combine_k routed rows never
+   * completes and its row of combine_out is not written.  0 = no combine.  Replaces the separate
+   * `reduce(y.view(T, k, -1), dim=1)` launch of tk/reduce.py:1143-1165 after the scatter of
+   * tk/matmul_details/_matmul.py:535-569. */
+  int32_t combine_k;
+  void* combine_out; /* bf16 [tokens, N], unit stride along N */
+  int64_t combine_stride_m;
+  int32_t* combine_counters;
 } tk_gemm_desc;
 
 #define TK_GEMM_TILE_COUNTER_WORDS 16
 
 /* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */
 int32_t tk_moe_gemm(const tk_gemm_desc* desc, tk_stream_t stream);
+
+/*
+ * GEMM with a ragged REDUCTION dimension (the expert weight gradient): for every slice e
+ *   y[e, m, n] = sum over k < slice_sizes[e] of a[m, a_slice_offs[e] + k] * b[b_slice_offs[e] + k, n]
+ * Replaces the `_matmul` launch of tk/matmul.py:659-726 when `b_ragged_metadata` is given (tk/matmul.py:376-384:
+ * ragged_dimension "K", batch = number of slices; kernel side tk/matmul_details/_matmul.py:252-272; torch statement
+ * tk/matmul.py:852-875).  The two operands carry their own slice offsets (one of them may be padded per slice); the
+ * sizes are those of b's metadata.  An empty slice yields a zero matrix.  No bias, gather, scatter or scales.
+ * a, b: TK_BF16 or TK_F16 (same type), any strides (in elements); fastest when the reduction index is the slow
+ * dimension of both (a = x^T, b = dy) with 16-byte aligned bases and strides that are multiples of 8.
+ * y: [n_slices, M, N], unit stride along N, TK_BF16 / TK_F16 / TK_F32; fp32 accumulation.
+ */
+typedef struct tk_ragged_k_desc {
+  const void* a;
+  int32_t dtype; /* of a and b */
+  int64_t a_stride_m, a_stride_k;
+  const void* b;
+  int64_t b_stride_k, b_stride_n;
+  void* y;
+  int32_t y_dtype;
+  int64_t y_stride_e, y_stride_m;
+  int32_t M, N, n_slices;
+  const int32_t* slice_sizes;  /* [n_slices] reduction length per slice */
+  const int32_t* a_slice_offs; /* [n_slices] first k of the slice in a */
+  const int32_t* b_slice_offs; /* [n_slices] first k of the slice in b */
+} tk_ragged_k_desc;
+
+int32_t tk_ragged_k_gemm(const tk_ragged_k_desc* desc, tk_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Element-wise companions of the GEMM

@@ -81,6 +81,30 @@ def matmul(x, w, bias, slice_sizes=None, gather_indx=None, scatter_indx=None, ga
     return out
 
 
+def matmul_ragged_k(a, b, sizes, a_offs, b_offs, out_dtype=None):
+    """out[e] = a[:, a_offs[e] : a_offs[e] + sizes[e]] @ b[b_offs[e] : b_offs[e] + sizes[e], :]   (matmul.py:852-875).
+
+    The reduction dimension is the ragged one: `a [M, Ka]`, `b [Kb, N]`, one `[M, N]` result per slice, zero for an
+    empty slice (matmul.py:860-861).  Each slice is an ordinary fp32-accumulated matmul (matmul.py:865-871 recurses
+    into the dense case without bias or scales); the reference collects the slices in an fp32 tensor, the kernel's
+    output type is `out_dtype` (default a's).
+    """
+    a = a.detach().to("cpu")
+    b = b.detach().to("cpu")
+    sizes = [int(v) for v in sizes.detach().to("cpu")]
+    a_offs = [int(v) for v in a_offs.detach().to("cpu")]
+    b_offs = [int(v) for v in b_offs.detach().to("cpu")]
+    out_dtype = out_dtype or a.dtype
+    out = torch.zeros((len(sizes), a.shape[0], b.shape[1]), dtype=out_dtype)
+    for e, k in enumerate(sizes):
+        if k == 0:
+            continue
+        xs = a[:, a_offs[e]:a_offs[e] + k].to(torch.float32)
+        ws = b[b_offs[e]:b_offs[e] + k, :].to(torch.float32)
+        out[e] = torch.matmul(xs, ws).to(out_dtype)
+    return out
+
+
 def swiglu(a: torch.Tensor, alpha: float, limit: float | None, out_dtype=None):
     """Interleaved (gate, linear) columns -> s*(linear+1), s = g*sigmoid(alpha*g)   (swiglu.py:89-100)."""
     a = a.detach().to("cpu")

@@ -381,3 +381,29 @@ def test_config5_full_shape_properties(api, device):
     perm = torch.randperm(T, generator=g)
     out_p, _, _ = _layer(api, dev, x[perm], logits[perm], k, w1t, None, w2t, None, pc(s1), pc(s2), fp8=True)
     assert torch.equal(out_p.cpu(), out.cpu()[perm]), "token permutation must permute the output rows exactly"
+
+
+@pytest.mark.parametrize("T", [1, 4, 16, 64])
+def test_fused_topk_combine_equals_reduce(api, device, gptoss_weights, T):
+    """`matmul_ogs(..., scatter_indx=...)` at decode shapes sums the k rows of every token inside the GEMM launch (the
+    wave that completes a token's rows last does it).  The result must equal `reduce` over the scattered rows bit for
+    bit (same fp32 sum in j order), on two calls in a row (the counters are left clean), and the layer built on it is
+    checked against the oracle."""
+    g = torch.Generator().manual_seed(5)
+    E, k, d = 128, 4, 2880
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g) + torch.randn((E, ), generator=g) * 1.5
+    W = gptoss_weights["tiled"]
+    rdata, gather, scatter = api.routing(logits.to(device), k)
+    pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
+    h = api.matmul(x.to(device), W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, precision_config=pc1,
+                   fused_activation=api.act(1.702, 7.0))
+    y = api.matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=scatter.dst_indx, precision_config=pc2, gammas=rdata.gate_scal)
+    want, _ = api.reduce(y.view(T, k, -1), dim=1)
+    for rep in range(2):
+        got = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=pc2, gammas=rdata.gate_scal)
+        assert got.shape == (T, d)
+        assert torch.equal(got, want), f"call {rep}: fused combine differs from reduce"
+    ref, _ = _oracle_layer_on_active_experts(x, logits, k, gptoss_weights["strided"])
+    assert_close(ref, got, maxtol=3e-2, what="layer output through the fused combine")
+    assert_allclose_gate(ref, got, what="layer output through the fused combine", max_bad_frac=LAYER_GATE_SLACK)

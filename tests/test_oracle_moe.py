@@ -198,3 +198,30 @@ def test_layer_gate_against_float64():
     # rounding the exact result once to bf16 is always inside the gate: the slack comes from the partial rows
     once = (exact.to(torch.bfloat16).double() - exact).abs() > (1e-2 + 2e-2 * exact.abs())
     assert int(once.sum()) == 0
+
+
+def test_ragged_k_is_a_masked_dense_product():
+    """Pins `matmul_ragged_k` by mathematics: with both operands' slices laid end to end at their offsets,
+    out[e][m][n] = sum_k a[m, ao_e + k] b[bo_e + k, n] is a float64 einsum over a 0/1 selector per slice; the offsets
+    of the two operands differ (one side padded), one slice is empty, and out[e] summed over e with equal offsets is
+    the plain product a @ b."""
+    g = torch.Generator().manual_seed(5)
+    sizes = torch.tensor([5, 0, 17, 32, 1], dtype=torch.int32)
+    a_offs = torch.tensor([0, 8, 8, 32, 64], dtype=torch.int32)   # padded to multiples of 8
+    b_offs = torch.tensor([0, 5, 5, 22, 54], dtype=torch.int32)   # dense
+    M, N = 9, 13
+    a = torch.randn((M, 72), generator=g).to(torch.bfloat16)
+    b = torch.randn((55, N), generator=g).to(torch.bfloat16)
+    got = omoe.matmul_ragged_k(a, b, sizes, a_offs, b_offs, out_dtype=torch.float32)
+    for e in range(5):
+        want = torch.zeros((M, N), dtype=torch.float64)
+        for kk in range(int(sizes[e])):
+            want += torch.outer(a[:, int(a_offs[e]) + kk].double(), b[int(b_offs[e]) + kk, :].double())
+        torch.testing.assert_close(got[e].double(), want, rtol=1e-5, atol=1e-5)
+    assert got[1].abs().max() == 0
+    # equal dense offsets: the slices partition K, so the outputs sum to the full product
+    got2 = omoe.matmul_ragged_k(a[:, :55], b, sizes, b_offs, b_offs, out_dtype=torch.float32)
+    torch.testing.assert_close(got2.sum(0).double(), a[:, :55].double() @ b.double(), rtol=1e-5, atol=1e-4)
+    # a transposed (strided) operand is the same problem
+    got3 = omoe.matmul_ragged_k(a.t().contiguous().t(), b, sizes, a_offs, b_offs, out_dtype=torch.float32)
+    assert torch.equal(got3, got)

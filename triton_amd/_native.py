@@ -65,6 +65,18 @@ class GemmDesc(_c.Structure):
         ("activation", _i32), ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
         ("w_layout", _i32), ("idle_cus", _i32), ("tile_counters", _ptr), ("x_rows", _i64),
         ("x_mx_scale", _ptr), ("xs_stride_m", _i64), ("y_mx_scale", _ptr), ("ys_stride_m", _i64),
+        ("combine_k", _i32), ("combine_out", _ptr), ("combine_stride_m", _i64), ("combine_counters", _ptr),
+    ]
+
+
+class RaggedKDesc(_c.Structure):
+    """struct tk_ragged_k_desc (field order and types follow include/triton_amd.h)."""
+    _fields_ = [
+        ("a", _ptr), ("dtype", _i32), ("a_stride_m", _i64), ("a_stride_k", _i64),
+        ("b", _ptr), ("b_stride_k", _i64), ("b_stride_n", _i64),
+        ("y", _ptr), ("y_dtype", _i32), ("y_stride_e", _i64), ("y_stride_m", _i64),
+        ("M", _i32), ("N", _i32), ("n_slices", _i32),
+        ("slice_sizes", _ptr), ("a_slice_offs", _ptr), ("b_slice_offs", _ptr),
     ]
 
 
@@ -80,6 +92,7 @@ SIGNATURES = {
     "tk_ragged_metadata": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _i64, _i32, _ptr]),
     "tk_ragged_remap": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32, _i32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
     "tk_moe_gemm": (_i32, [_c.POINTER(GemmDesc), _ptr]),
+    "tk_ragged_k_gemm": (_i32, [_c.POINTER(RaggedKDesc), _ptr]),
     "tk_swiglu": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _f32, _f32, _i32, _ptr, _ptr]),
     "tk_reduce_mid": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "tk_reduce_mid_backward": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),

@@ -43,6 +43,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+// byte offset that a buffer resource drops (stores) or reads as zero (loads): buffers span less than 2 GiB (host check)
+constexpr uint32_t kDroppedStore = 0x80000000u;
 typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
 
 enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3
@@ -86,6 +89,10 @@ struct GemmParams {
   int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
   int32_t* tile_counters;  // persistent kernels: kTileCounterWords zeroed words for dynamic tile claiming, or null
   uint32_t y_bytes;        // persistent MXFP4 kernels: bytes of the output buffer that rows may be written to (< 2 GiB)
+  int32_t combine_k;          // decode kernel: > 0 = sum the k rows of every token into combine_out (fused top-k combine)
+  uint16_t* combine_out;      // bf16 [tokens, N]
+  int64_t combine_stride;
+  int32_t* combine_counters;  // zeroed [tokens * ceil(N / 32)] words, left zero
   const uint8_t* x_mx_scale;  // e8m0 block scales of MXFP8 activations [rows, K/32], or null
   int64_t xs_stride_m;
   uint8_t* y_mx_scale;        // e8m0 block scales of an MXFP8 output [rows, N_out/32], or null
@@ -740,8 +747,6 @@ constexpr int kMetaSlices = 1024;
 // beyond the buffer resource's range, which the hardware drops.  With no branch around a store the number of
 // stores between two loads is the same on every path, so the compiler's vmcnt waits for loads issued BEFORE the
 // epilogue (the next unit's first operands) do not wait for these stores to drain.
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-constexpr uint32_t kDroppedStore = 0x80000000u;  // output buffers span less than 2 GiB (checked by the host)
 
 template <int G, int MFW, int NFW, bool SWIGLU>
 __device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc, const float* bias_s,
@@ -1264,11 +1269,91 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 // one stage ahead left their latency exposed), and issues 16x16x32 MFMAs
 // transposed like the prefill kernel (lane = column, 4 k-groups).  Within a stage lane group kg owns
 // k in [kg*32, kg*32 + 32): exactly one MX block and one 16-byte piece of the tiled layout.
-template <int MR, bool SWIGLU>
+// Epilogue of the decode kernel with the top-k combine fused behind the scatter (the reference runs `reduce` over the k
+// rows of every token as a launch of its own, reduce.py:1143-1165).  The k rows of token t are written by up to k
+// different waves, anywhere on the chip; each counts itself in at counter (t, fragment) once its rows have reached
+// memory, and the wave that arrives last sums the k rows in their order j = 0..k-1 in fp32, exactly as the
+// stand-alone kernel does, writes the token's row of the result and clears the counter for the next launch.
+// The eight XCDs have an L2 each, so rows that another XCD will read go around it: stores and loads of y carry the
+// sc0 sc1 cache policy (write-through to memory / read from memory) and the counter is a device-scope atomic; the
+// alternative, a device-scope release fence per wave, writes back and invalidates a whole L2 each time and more than
+// doubled the kernel's time.  acc[g][j][i]: sub-fragment g (columns F*32 + g*16 + kg*4 + i), row fragment j.
+template <int MR>
+__device__ __forceinline__ void combine_epilogue(const GemmParams& p, f32x4_t (&acc)[2][MR], int expert, int off_m, int start_m, int eM, int F,
+                                                 int nfr, int lr, int kg) {
+  constexpr int kThrough = 1 | 16;  // aux bits of the buffer instructions: sc0 | sc1
+  const int N = p.N, k = p.combine_k;
+  const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
+  const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
+  float b4[2][4];
+#pragma unroll
+  for (int g = 0; g < 2; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = F * 32 + g * 16 + kg * 4 + i;
+      b4[g][i] = (p.bias && n < N) ? load_scalar(p.bias, (int64_t)expert * p.bias_stride_e + n, p.bias_is_f32) : 0.f;
+    }
+  int token[MR];
+#pragma unroll
+  for (int j = 0; j < MR; ++j) {
+    const int row = off_m + j * 16 + lr;
+    const bool ok = row < eM;
+    const int srow = start_m + (ok ? row : eM - 1);
+    const float gam = p.gammas ? load_scalar(p.gammas, srow, p.gammas_is_f32) : 1.0f;
+    int dst = srow < p.scatter_len ? p.scatter[srow] : -1;
+    dst = ok ? dst : -1;
+    token[j] = dst >= 0 ? dst / k : -1;
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int n0 = F * 32 + g * 16 + kg * 4;
+      const u32x2_t w = {pack_bf16x2((acc[g][j][0] + b4[g][0]) * gam, (acc[g][j][1] + b4[g][1]) * gam),
+                         pack_bf16x2((acc[g][j][2] + b4[g][2]) * gam, (acc[g][j][3] + b4[g][3]) * gam)};
+      const uint32_t off = (dst >= 0 && n0 < N) ? (uint32_t)dst * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
+      __builtin_amdgcn_raw_buffer_store_b64(w, yrsrc, off, 0, kThrough);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows have reached memory before it is counted
+#pragma unroll
+  for (int j = 0; j < MR; ++j) {
+    int seen = -1;
+    if (kg == 0 && token[j] >= 0)
+      seen = __hip_atomic_fetch_add(&p.combine_counters[(int64_t)token[j] * nfr + F], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    seen = __shfl(seen, lr);  // the row's four lanes (lr, lr + 16, ...) share lane lr's count
+    const bool last = token[j] >= 0 && seen == k - 1;
+    // (the loads below depend on the atomic's result, so they cannot be issued before it has been performed)
+    const uint32_t base = last ? (uint32_t)(token[j] * k) * row_bytes : kDroppedStore;
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int n0 = F * 32 + g * 16 + kg * 4;
+      float sum[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int jj = 0; jj < k; ++jj) {
+        const uint32_t off = (last && n0 < N) ? base + (uint32_t)jj * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
+        const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(yrsrc, off, 0, kThrough);  // out-of-range lanes read zero
+        sum[0] += bits_f32(v.x << 16);
+        sum[1] += bits_f32(v.x & 0xFFFF0000u);
+        sum[2] += bits_f32(v.y << 16);
+        sum[3] += bits_f32(v.y & 0xFFFF0000u);
+      }
+      if (last && n0 < N) {
+        uint16_t* o = p.combine_out + (int64_t)token[j] * p.combine_stride + n0;
+        if (n0 + 4 <= N && (p.combine_stride & 3) == 0) {
+          *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]));
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) o[i] = f32_to_bf16_bits(sum[i]);
+        }
+      }
+    }
+    if (last && kg == 0) __hip_atomic_store(&p.combine_counters[(int64_t)token[j] * nfr + F], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int MR, int NFD, bool SWIGLU>
 __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   typedef Frag<16> FR;
   constexpr int WDD = 4, XDD = 4;  // ring depths (stages) of the weight / activation registers (both run 3 stages ahead)
-  __shared__ float red[3][2 * MR * 4][64];  // K-split partial sums of waves 1..3
+  __shared__ float red[3][NFD * 2 * MR * 4][64];  // K-split partial sums of waves 1..3
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1276,16 +1361,19 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   const int K = p.K, N = p.N;
   const int nst = p.w_nst;
   const int nfr = (N + 31) >> 5;
+  // A wave owns NFD neighbouring 32-column fragments of one row block: the activations it fetches (twice the bytes of a
+  // fragment's weights per stage) then feed NFD fragments' MFMAs.
+  const int nslot = (nfr + NFD - 1) / NFD;  // fragment groups per row block
 
-  // K-split: when few tiles are live (a handful of active experts), 2 or 4 waves share a fragment and take
+  // K-split: when few tiles are live (a handful of active experts), 2 or 4 waves share a fragment group and take
   // every 2nd / 4th K-stage each, so that enough loads are in flight to cover the HBM latency.  The factor is
   // derived on the device from the live block count (the host never reads it) and is uniform over the grid;
   // the grid is launched for the largest factor and the surplus workgroups leave at once.
   const int nblk = p.slice_sizes ? p.block_offs[p.n_slices] : p.total_tiles;
-  const int frag_tiles = nblk * nfr;  // (row block, fragment) pairs = waves at split 1
+  const int frag_tiles = nblk * nslot;  // (row block, fragment group) pairs = waves at split 1
   const int ksplit = frag_tiles <= 1024 ? 4 : (frag_tiles <= 2048 ? 2 : 1);
-  const int fpw = 4 / ksplit;                        // fragments per workgroup
-  const int grid_n = (nfr + fpw - 1) / fpw;          // workgroups per row block
+  const int fpw = 4 / ksplit;                        // fragment groups per workgroup
+  const int grid_n = (nslot + fpw - 1) / fpw;        // workgroups per row block
   if ((int)blockIdx.x >= nblk * grid_n) return;
   const int pid_n = blockIdx.x % grid_n, pid_m = blockIdx.x / grid_n;
   const int kslice = wave % ksplit;
@@ -1302,17 +1390,29 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     start_m = 0;
     eM = p.M;
   }
-  int F = pid_n * fpw + wave / ksplit;  // this wave's 32-column fragment
-  const bool live_wave = F < nfr;
-  F = live_wave ? F : nfr - 1;
+  const int slot = pid_n * fpw + wave / ksplit;  // this wave's fragment group
+  const bool live_wave = slot < nslot;
+  int F[NFD];
+  bool live_f[NFD];
+#pragma unroll
+  for (int fd = 0; fd < NFD; ++fd) {
+    const int f = (live_wave ? slot : nslot - 1) * NFD + fd;
+    live_f[fd] = live_wave && f < nfr;
+    F[fd] = f < nfr ? f : nfr - 1;
+  }
   const int rows = (eM - off_m) < MR * 16 ? (eM - off_m) : MR * 16;
   const int nj = (rows + 15) >> 4;  // row fragments with valid rows (1..MR)
   // this wave's stages: kslice, kslice + ksplit, ...
   const int my_nst = (nst - kslice + ksplit - 1) / ksplit;
 
   // weights: sub-fragment g holds columns F*32 + g*16 + lr; this lane's piece of a stage is k-block kg
-  const uint8_t* wbase = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F * nst * 2048 + (kg & 1) * 1024 + ((kg >> 1) * 32 + lr) * 16;
-  const uint8_t* sbase = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)F * nst * 128 + lr * 4;
+  const uint8_t* wbase[NFD];
+  const uint8_t* sbase[NFD];
+#pragma unroll
+  for (int fd = 0; fd < NFD; ++fd) {
+    wbase[fd] = p.w + (int64_t)expert * p.w_stride_e + (int64_t)F[fd] * nst * 2048 + (kg & 1) * 1024 + ((kg >> 1) * 32 + lr) * 16;
+    sbase[fd] = p.w_scale + (int64_t)expert * p.ws_stride_e + (int64_t)F[fd] * nst * 128 + lr * 4;
+  }
   // activations: row j*16 + lr, 64 bytes per stage at k offset kg*32
   const uint8_t* xptr[MR];
 #pragma unroll
@@ -1323,16 +1423,18 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     xptr[j] = p.x + src * p.x_stride_m * 2;
   }
 
-  typename FR::acc_t acc[2][MR];
+  typename FR::acc_t acc[NFD][2][MR];
 #pragma unroll
-  for (int g = 0; g < 2; ++g)
+  for (int fd = 0; fd < NFD; ++fd)
 #pragma unroll
-    for (int j = 0; j < MR; ++j)
+    for (int g = 0; g < 2; ++g)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[g][j][i] = 0.f;
+      for (int j = 0; j < MR; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[fd][g][j][i] = 0.f;
 
-  u32x4_t wr[WDD][2];
-  uint32_t sr[WDD][2];
+  u32x4_t wr[WDD][NFD][2];
+  uint32_t sr[WDD][NFD][2];
   u32x4_t xr[XDD][MR][4];
 
   // `i` counts this wave's own stages; the global stage is kslice + i*ksplit (clamped: surplus loads re-read
@@ -1342,10 +1444,12 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     int s = kslice + i * ksplit;
     s = s < nst ? s : nst - 1;
 #pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      wr[SL][g] = *reinterpret_cast<const u32x4_t*>(wbase + (int64_t)s * 2048 + g * 256);
-      sr[SL][g] = *reinterpret_cast<const uint32_t*>(sbase + (int64_t)s * 128 + g * 64);
-    }
+    for (int fd = 0; fd < NFD; ++fd)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        wr[SL][fd][g] = *reinterpret_cast<const u32x4_t*>(wbase[fd] + (int64_t)s * 2048 + g * 256);
+        sr[SL][fd][g] = *reinterpret_cast<const uint32_t*>(sbase[fd] + (int64_t)s * 128 + g * 64);
+      }
   };
   auto load_x = [&](auto slot_c, int i) __attribute__((always_inline)) {
     constexpr int SL = decltype(slot_c)::value;
@@ -1364,19 +1468,23 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     constexpr int XS = decltype(xslot_c)::value;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      bf16x8_t wf[2];
+      bf16x8_t wf[NFD][2];
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        const u32x4_t v = wr[WS][g];
-        const uint32_t raw = t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
-        wf[g] = dequant8(raw, bits_f32(((sr[WS][g] >> (8 * kg)) & 0xFFu) << 23));
-      }
+      for (int fd = 0; fd < NFD; ++fd)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const u32x4_t v = wr[WS][fd][g];
+          const uint32_t raw = t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
+          wf[fd][g] = dequant8(raw, bits_f32(((sr[WS][fd][g] >> (8 * kg)) & 0xFFu) << 23));
+        }
 #pragma unroll
       for (int j = 0; j < MR; ++j) {
         if (j < nj) {
           const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xr[XS][j][t]);
 #pragma unroll
-          for (int g = 0; g < 2; ++g) acc[g][j] = FR::mma(wf[g], xf, acc[g][j]);
+          for (int fd = 0; fd < NFD; ++fd)
+#pragma unroll
+            for (int g = 0; g < 2; ++g) acc[fd][g][j] = FR::mma(wf[fd][g], xf, acc[fd][g][j]);
         }
       }
     }
@@ -1408,27 +1516,40 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     });
   }
   if (ksplit > 1) {
-    // sum the K-slices of a fragment in the wave with kslice 0 (through LDS), which then runs the epilogue
+    // sum the K-slices of a fragment group in the wave with kslice 0 (through LDS), which then runs the epilogue
     if (kslice != 0) {
 #pragma unroll
-      for (int g = 0; g < 2; ++g)
+      for (int fd = 0; fd < NFD; ++fd)
 #pragma unroll
-        for (int j = 0; j < MR; ++j)
+        for (int g = 0; g < 2; ++g)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) red[wave - 1][(g * MR + j) * 4 + i][lane] = acc[g][j][i];
+          for (int j = 0; j < MR; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave - 1][((fd * 2 + g) * MR + j) * 4 + i][lane] = acc[fd][g][j][i];
     }
     __syncthreads();
     if (kslice != 0) return;
     for (int o = 1; o < ksplit; ++o)
 #pragma unroll
-      for (int g = 0; g < 2; ++g)
+      for (int fd = 0; fd < NFD; ++fd)
 #pragma unroll
-        for (int j = 0; j < MR; ++j)
+        for (int g = 0; g < 2; ++g)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[g][j][i] += red[wave + o - 1][(g * MR + j) * 4 + i][lane];
+          for (int j = 0; j < MR; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[fd][g][j][i] += red[wave + o - 1][((fd * 2 + g) * MR + j) * 4 + i][lane];
   }
-  if (live_wave)
-    gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc, expert, off_m, start_m, eM, F * 32, F * 32 + 32 <= N, 0, lr, kg);
+#pragma unroll
+  for (int fd = 0; fd < NFD; ++fd) {
+    if (!live_f[fd]) continue;
+    if constexpr (!SWIGLU) {
+      if (p.combine_k > 0) {
+        combine_epilogue<MR>(p, acc[fd], expert, off_m, start_m, eM, F[fd], nfr, lr, kg);
+        continue;
+      }
+    }
+    gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc[fd], expert, off_m, start_m, eM, F[fd] * 32, F[fd] * 32 + 32 <= N, 0, lr, kg);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2094,19 +2215,27 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8n_kernel(const GemmParams p) 
   }  // rounds
 }
 
-template <int MR>
-int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
+template <int MR, int NFD>
+int32_t launch_mxd_n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
   GemmParams q = p;
   q.total_tiles = grid_m;  // row blocks in the non-ragged case
-  // sized for a K-split of 4 (one fragment per workgroup); with a smaller split the surplus leaves at once
-  const int64_t grid = (int64_t)grid_m * cdiv(p.N, 32);
+  // sized for a K-split of 4 (one fragment group per workgroup); with a smaller split the surplus leaves at once
+  const int64_t grid = (int64_t)grid_m * cdiv(cdiv(p.N, 32), NFD);
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   if (swiglu)
-    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, true>), dim3((unsigned)grid), dim3(256), 0, st, q);
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, true>), dim3((unsigned)grid), dim3(256), 0, st, q);
   else
-    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, false>), dim3((unsigned)grid), dim3(256), 0, st, q);
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, false>), dim3((unsigned)grid), dim3(256), 0, st, q);
   return check_launch("moe_gemm_mxd_kernel");
+}
+template <int MR>
+int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
+  // Two fragments per wave halve the activation reads (which come from L2) at the price of half as many waves.  With
+  // few rows only a few experts are live and the kernel needs every wave it can get to keep HBM busy; from about a
+  // hundred rows on the activation traffic is what limits it.  (Measured at 128 experts, top-4: 16 tokens are 6 %
+  // faster with one fragment, 64 tokens 8 % faster with two.)
+  return p.M >= 128 ? launch_mxd_n<MR, 2>(p, grid_m, swiglu, st) : launch_mxd_n<MR, 1>(p, grid_m, swiglu, st);
 }
 
 // Raises a kernel's dynamic LDS limit above 64 KiB, once per (kernel, device): the table is keyed on the kernel's
@@ -2338,6 +2467,25 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.idle_cus = d->idle_cus;
   p.tile_counters = d->tile_counters;
   p.y_bytes = 0;
+  p.combine_k = 0;
+  p.combine_out = nullptr;
+  p.combine_stride = 0;
+  p.combine_counters = nullptr;
+  if (d->combine_k > 0) {
+    if (!(d->w_layout == TK_W_TILED && d->w_dtype == TK_E2M1 && (d->block_m == 16 || d->block_m == 32)))
+      return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine needs tiled MXFP4 weights and block_m 16 or 32");
+    if (!d->scatter_indx || !d->combine_out || !d->combine_counters || d->activation != TK_ACT_NONE)
+      return fail(TK_ERR_INVALID, "tk_moe_gemm: the fused top-k combine needs scatter_indx, combine_out and combine_counters, and no activation");
+    if (d->scatter_len % d->combine_k) return fail(TK_ERR_INVALID, "tk_moe_gemm: scatter_len %d is not a multiple of combine_k %d", d->scatter_len, d->combine_k);
+    const int64_t yb = (int64_t)d->scatter_len * d->y_stride_m * 2;
+    if (yb >= (int64_t)1 << 31 || d->y_stride_m % 4 || (reinterpret_cast<uintptr_t>(d->y) & 7) || d->N % 4)
+      return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine needs N %% 4 == 0 and 8-byte aligned output rows spanning less than 2 GiB");
+    p.y_bytes = (uint32_t)yb;
+    p.combine_k = d->combine_k;
+    p.combine_out = static_cast<uint16_t*>(d->combine_out);
+    p.combine_stride = d->combine_stride_m;
+    p.combine_counters = d->combine_counters;
+  }
   p.x_mx_scale = static_cast<const uint8_t*>(d->x_mx_scale);
   p.xs_stride_m = d->xs_stride_m;
   p.y_mx_scale = static_cast<uint8_t*>(d->y_mx_scale);

@@ -66,7 +66,8 @@ def matmul_ogs(x, w, bias, routing_data: RoutingData | None = None, gather_indx:
                scatter_indx: ScatterIndx | None = None, precision_config: PrecisionConfig | None = None, betas=None,
                gammas=None, fused_activation: FusedActivation | None = None, **kwargs):
     """`matmul` over the experts of `routing_data`; with `scatter_indx` the k expert rows of every token
-    are summed, so the result has one row per token."""
+    are summed, so the result has one row per token.  At decode shapes (tiled MXFP4 weights, a few rows per expert) the
+    sum happens inside the GEMM launch; otherwise `reduce` follows it."""
     md = routing_data.expt_data if routing_data is not None else None
     g = None
     if gather_indx is not None:
@@ -76,10 +77,13 @@ def matmul_ogs(x, w, bias, routing_data: RoutingData | None = None, gather_indx:
         else:
             g = torch.div(gather_indx.src_indx, k, rounding_mode="trunc").to(torch.int32)
     s = scatter_indx.dst_indx if scatter_indx is not None else None
+    k = routing_data.n_expts_act if (routing_data is not None and scatter_indx is not None) else None
     y = matmul(x, w, bias, md, gather_indx=g, scatter_indx=s, precision_config=precision_config, betas=betas,
-               gammas=gammas, fused_activation=fused_activation, **kwargs)
+               gammas=gammas, fused_activation=fused_activation, _combine_k=k, **kwargs)
     if scatter_indx is None:
         return y
-    k = routing_data.n_expts_act
+    combined = getattr(y, "_tk_combined", None)
+    if combined is not None:  # decode shapes: the GEMM's last wave per token has already summed its k rows
+        return combined
     out, _ = reduce(y.view(y.shape[0] // k, k, y.shape[-1]), dim=1)
     return out

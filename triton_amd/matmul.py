@@ -11,8 +11,7 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
     bf16         mxfp4 (uint8 e2m1 + e8m0)      dequantised in registers, bf16 MFMA, fp32 accumulate
     fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
 
-Options of the reference signature that this build rejects with NotImplementedError: ragged-K
-(`b_ragged_metadata`), `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
+Options of the reference signature that this build rejects with NotImplementedError: `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
 output / accumulator scales, batched 3-D activations, split-k.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
 `flex_ctx.rhs_data.scale`) are folded into the per-row / per-column scales of the epilogue.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
 MX quantiser kernel on the same stream.
@@ -120,6 +119,21 @@ def _tile_counters(device: torch.device) -> torch.Tensor:
     return buf
 
 
+_COMBINE_COUNTERS: dict = {}
+_COMBINE_COUNTER_WORDS = 1 << 16
+
+
+def _combine_counters(device: torch.device) -> torch.Tensor:
+    """Zeroed int32 words for the fused top-k combine (`tk_gemm_desc.combine_counters`), one buffer per (device, stream)
+    like the tile counters; the kernel leaves them zero."""
+    key = (device.index, nt.stream_ptr(device))
+    buf = _COMBINE_COUNTERS.get(key)
+    if buf is None:
+        buf = torch.zeros(_COMBINE_COUNTER_WORDS, dtype=torch.int32, device=device)
+        _COMBINE_COUNTERS[key] = buf
+    return buf
+
+
 def _flex_out_is_trivial(flex: FlexCtx) -> bool:
     return (flex.acc_data.scale is None and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
             and flex.out_data.checksum_scale is None)
@@ -205,20 +219,86 @@ def _localise_remapped_metadata(md: RaggedTensorMetadata, n_local: int, n_rows: 
     return RaggedTensorMetadata(sizes, md.slice_offs[:n_local + 1], local.block_offs_data, local.block_schedule_data)
 
 
+def _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_indx, scatter_indx, precision_config, betas,
+                     gammas, out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in):
+    """The reduction dimension is ragged (triton_kernels/matmul.py:376-384): one [M, N] output per slice,
+    out[e] = a[:, xo[e] : xo[e] + k_e] @ b[wo[e] : wo[e] + k_e, :] with k_e = b_ragged_metadata.slice_sizes[e], xo / wo the
+    slice offsets of a's and b's metadata (torch statement: triton_kernels/matmul.py:852-875).  This is the expert
+    weight gradient dW[e] = x_e^T @ dy_e.  Dense bf16 / fp16 operands only; no bias (the reference's own test passes
+    none for this mode, tests/test_matmul.py:469), gather, scatter, scales or epilogue."""
+    assert gather_indx is None and scatter_indx is None  # triton_kernels/matmul.py:279-281
+    if a_ragged_metadata is None:
+        raise ValueError("ragged-K matmul needs a_ragged_metadata as well (the slice offsets of a along K)")
+    for what, v in (("bias", bias), ("betas", betas), ("gammas", gammas), ("out_alpha", out_alpha), ("fused_comm", fused_comm),
+                    ("c_acc_in", c_acc_in)):
+        if v is not None:
+            raise NotImplementedError(f"{what} is not supported with b_ragged_metadata")
+    if fused_activation is not None and fused_activation.specs.fn is not None:
+        raise NotImplementedError("a fused activation is not supported with b_ragged_metadata")
+    if epilogue is not None and (epilogue.specs.fn is not None or epilogue.specs.name != "dflt"):
+        raise NotImplementedError("an epilogue is not supported with b_ragged_metadata")
+    pc = precision_config or PrecisionConfig()
+    if pc.a_mx_scale is not None or pc.b_mx_scale is not None or pc.c_mx_scale is not None:
+        raise NotImplementedError("MX operands are not supported with b_ragged_metadata")
+    if not (_flex_out_is_trivial(pc.flex_ctx) and pc.flex_ctx.lhs_data.scale is None and pc.flex_ctx.rhs_data.scale is None):
+        raise NotImplementedError("flexpoint scales are not supported with b_ragged_metadata")
+    if isinstance(a, Tensor):
+        a = a.storage.data
+    if isinstance(b, Tensor):
+        if not isinstance(b.storage.layout, StridedLayout):
+            raise NotImplementedError(f"weight layout {type(b.storage.layout).__name__} is not supported with b_ragged_metadata")
+        b = b.storage.data
+    if a.ndim != 2 or b.ndim != 2:
+        raise NotImplementedError("ragged-K matmul takes 2-D operands")
+    nt.require_gpu(a, "a")
+    if a.dtype != b.dtype or a.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError(f"ragged-K matmul takes bf16 or fp16 operands of one type (got {a.dtype} and {b.dtype})")
+    out_dtype = pc.out_dtype or a.dtype
+    if out_dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError(f"output dtype {out_dtype} is not supported with b_ragged_metadata")
+    n_slices = b_ragged_metadata.n_slices
+    assert a_ragged_metadata.n_slices == n_slices
+    M, N = a.shape[0], b.shape[1]
+    if c is None:
+        c = torch.empty((n_slices, M, N), dtype=out_dtype, device=a.device)
+    else:
+        assert c.shape == (n_slices, M, N) and c.dtype == out_dtype and (N == 0 or c.stride(-1) == 1)
+    d = nt.RaggedKDesc()
+    d.a, d.dtype = a.data_ptr(), nt.TORCH_TO_TK[a.dtype]
+    d.a_stride_m, d.a_stride_k = a.stride(0), a.stride(1)
+    d.b = b.data_ptr()
+    d.b_stride_k, d.b_stride_n = b.stride(0), b.stride(1)
+    d.y, d.y_dtype = c.data_ptr(), nt.TORCH_TO_TK[out_dtype]
+    d.y_stride_e, d.y_stride_m = c.stride(0), c.stride(1)
+    d.M, d.N, d.n_slices = M, N, n_slices
+    sizes, a_offs, b_offs = b_ragged_metadata.slice_sizes, a_ragged_metadata.slice_offs, b_ragged_metadata.slice_offs
+    assert sizes.dtype == a_offs.dtype == b_offs.dtype == torch.int32
+    assert sizes.is_contiguous() and a_offs.is_contiguous() and b_offs.is_contiguous()
+    d.slice_sizes, d.a_slice_offs, d.b_slice_offs = sizes.data_ptr(), a_offs.data_ptr(), b_offs.data_ptr()
+    with nt.on_device(a.device):
+        nt.check(nt.lib().tk_ragged_k_gemm(d, nt.stream_ptr(a.device)), "tk_ragged_k_gemm")
+    return c
+
+
 def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
            b_ragged_metadata: RaggedTensorMetadata | None = None, gather_indx: torch.Tensor | None = None,
            scatter_indx: torch.Tensor | None = None, precision_config: PrecisionConfig | None = None,
            betas: torch.Tensor | None = None, gammas: torch.Tensor | None = None, out_alpha: float | None = None,
            c: torch.Tensor | None = None, fused_comm: FusedComm | None = None,
            fused_activation: FusedActivation | None = None, epilogue: Epilogue | None = None,
-           c_acc_in: torch.Tensor | None = None):
+           c_acc_in: torch.Tensor | None = None, *, _combine_k: int | None = None):
     """
     Y[:, :] = 0
     for e in experts:
         Y[idxs_y_m(e), :] += matmul(X[idxs_x_m(e), :], W[e, :, :])
+
+    `_combine_k` (used by `legacy.matmul_ogs`, not part of the reference's signature): with `scatter_indx` mapping rows
+    to flat positions t * k + j, the decode kernel may also sum the k rows of every token; the result is then attached to
+    the returned tensor as `._tk_combined` ([tokens, N]) and the caller skips its `reduce`.
     """
     if b_ragged_metadata is not None:
-        raise NotImplementedError("ragged-K matmul (b_ragged_metadata) is a training feature and is not supported")
+        return _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_indx, scatter_indx, precision_config,
+                                betas, gammas, out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in)
     if c_acc_in is not None:
         raise NotImplementedError("c_acc_in is not supported")
     if fused_comm is not None:
@@ -504,6 +584,15 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if c_scale is not None:
         d.y_mx_scale = c_scale.data_ptr()
         d.ys_stride_m = c_scale.stride(-2)
+    combined = None
+    if (_combine_k and tiled and not mx_act and block_m <= 32 and act == nt.TK_ACT_NONE and scatter_indx is not None
+            and scatter_indx.shape[0] % _combine_k == 0
+            and (scatter_indx.shape[0] // _combine_k) * ((N + 31) // 32) <= _COMBINE_COUNTER_WORDS):
+        combined = torch.empty((scatter_indx.shape[0] // _combine_k, N), dtype=c.dtype, device=c.device)
+        d.combine_k = int(_combine_k)
+        d.combine_out = combined.data_ptr()
+        d.combine_stride_m = combined.stride(0)
+        d.combine_counters = _combine_counters(a.device).data_ptr()
     if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES and not mx_act:
         d.tile_counters = _tile_counters(a.device).data_ptr()
     with nt.on_device(a.device):
@@ -511,4 +600,6 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     del keep
     if y_buf is not c:
         c.copy_(y_buf)
+    if combined is not None:
+        c._tk_combined = combined
     return c
