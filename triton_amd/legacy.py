@@ -87,3 +87,6 @@ def matmul_ogs(x, w, bias, routing_data: RoutingData | None = None, gather_indx:
         return combined
     out, _ = reduce(y.view(y.shape[0] // k, k, y.shape[-1]), dim=1)
     return out
+
+
+from .torch_twins import matmul_ogs_torch, routing_torch  # noqa: E402,F401  (reference twins)

@@ -603,3 +603,6 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if combined is not None:
         c._tk_combined = combined
     return c
+
+
+from .torch_twins import matmul_torch  # noqa: E402,F401  (reference twin; never called by `matmul`)

@@ -172,3 +172,6 @@ def upcast_from_mxfp(tensor: torch.Tensor, scale: torch.Tensor, target_dtype: to
         shp = (1, ) * out.ndim if tensor_scale.numel() == 1 else (*tensor_scale.shape[:axis], 1, *tensor_scale.shape[axis:])
         out = out * tensor_scale.to(device=out.device).reshape(shp)
     return out
+
+
+from ..torch_twins import downcast_to_mxfp_torch, upcast_from_mxfp_torch  # noqa: E402,F401  (reference twins)

@@ -122,3 +122,6 @@ def _reduce_forward(x, mask, scale, y):
             nt.lib().tk_reduce_mid(x.data_ptr(), nt.TORCH_TO_TK[x.dtype], A, K, C, x.stride(0), x.stride(1), m_ptr, *ms, s_ptr,
                                    *ss, y.data_ptr(), y.stride(0) if A else 0, nt.stream_ptr(x.device)))
     return y, None
+
+
+from .torch_twins import reduce_torch  # noqa: E402,F401  (reference twin; never called by `reduce`)

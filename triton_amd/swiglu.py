@@ -62,3 +62,6 @@ def swiglu(a, alpha, precision_config, routing_data=None):
                                out.stride(0), float(alpha), float(limit) if limit is not None else 0.0,
                                int(limit is not None), nt.ptr(n_tokens), nt.stream_ptr(a.device)))
     return out.view(a.shape[:-1] + out.shape[-1:])
+
+
+from .torch_twins import swiglu_torch  # noqa: E402,F401  (reference twin; never called by `swiglu`)

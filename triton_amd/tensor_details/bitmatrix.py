@@ -109,3 +109,11 @@ def make_bitmatrix_metadata(nonzero_indx, bitmatrix):
                vals=None, bitmatrix_data=None, want_meta=True)
     return BitmatrixMetadata(col_sum=r["col_sum"], col_sorted_indx=r["col_sorted_indx"],
                              row_sorted_indx=r["row_sorted_indx"])
+
+
+def __getattr__(name):
+    # the reference's torch twin of this module, resolved on first use (it needs the fully imported `tensor` module)
+    if name == "make_bitmatrix_metadata_torch":
+        from .. import torch_twins
+        return getattr(torch_twins, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

@@ -120,3 +120,11 @@ def remap_ragged_tensor_metadata(src_ragged_tensor_metadata: RaggedTensorMetadat
     out = RaggedTensorMetadata(slice_sizes, offs[0], offs[1:], sched)
     out.remapped_from = n_slices  # tells `matmul` that block offsets are those of the source tensor, not a running sum
     return out
+
+
+def __getattr__(name):
+    # the reference's torch twin of this module, resolved on first use (it needs the fully imported `tensor` module)
+    if name == "make_ragged_tensor_metadata_torch":
+        from .. import torch_twins
+        return getattr(torch_twins, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

@@ -126,3 +126,6 @@ def topk(x: Union[Tensor, torch.Tensor], k: int, apply_softmax: bool = True, dim
     meta = BitmatrixMetadata(col_sum=r["col_sum"], col_sorted_indx=r["col_sorted_indx"],
                              row_sorted_indx=r["row_sorted_indx"])
     return SparseMatrix(vals=y_vals, indx=y_indx, mask=mask, mask_metadata=meta)
+
+
+from .torch_twins import topk_torch  # noqa: E402,F401  (reference twin; never called by `topk`)
