@@ -222,6 +222,26 @@ def bench_mx(device, steps, warmup):
                 frac_hbm_dequant=round(nbytes / ms_d / 1e6 / PEAK_HBM_GBPS, 4))
 
 
+def bench_ragged_k(device, steps, warmup):
+    """Expert weight gradient of config 3's first GEMM: dW1[e] = x_e^T @ dh_e for 128 experts, 16384 routed rows,
+    [2880, 5760] per expert in bf16 (bound by writing the 4.2 GB of gradients)."""
+    from triton_kernels.matmul import matmul
+    from triton_kernels.tensor import make_ragged_tensor_metadata
+    E, R, d, f2 = 128, 16384, 2880, 5760
+    g = torch.Generator().manual_seed(6)
+    cuts = torch.sort(torch.randint(0, R + 1, (E - 1, ), generator=g)).values
+    sizes = torch.diff(torch.cat([torch.tensor([0]), cuts, torch.tensor([R])])).to(torch.int32).to(device)
+    md = make_ragged_tensor_metadata(sizes, R)
+    x = torch.randn((R, d), device=device).to(torch.bfloat16)
+    dh = torch.randn((R, f2), device=device).to(torch.bfloat16)
+    out = torch.empty((E, d, f2), dtype=torch.bfloat16, device=device)
+    ms = time_steps(lambda: matmul(x.t(), dh, None, a_ragged_metadata=md, b_ragged_metadata=md, c=out), steps, warmup)
+    nbytes = out.numel() * 2 + x.numel() * 2 + dh.numel() * 2
+    flops = 2.0 * R * d * f2
+    return dict(ms=round(ms, 4), GBps=round(nbytes / ms / 1e6, 1), frac_hbm=round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4),
+                TFLOPs=round(flops / ms / 1e9, 1))
+
+
 def bench_fp8(device, steps, warmup):
     """Config 5 (Mixtral-style FP8) at full size: 8192 tokens, top-2 of 8 experts, W1 [8, 4096, 28672] and
     W2 [8, 14336, 4096] in e4m3 with per-output-channel fp32 scales, activations quantised per token to e4m3
@@ -317,6 +337,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the decode and MX round-trip figures")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run a 1 GiB device copy (reference kernel for counter runs)")
+    ap.add_argument("--only", choices=["mx", "decode", "fp8", "ragged_k"],
+                    help="run one of the side workloads alone and print its figures (for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (with more GPUs the layer shards by expert, which is not built)",
@@ -327,6 +349,12 @@ def main():
         sys.exit(2)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.only:
+        if args.calibrate_copy:
+            calibration_copy(device)
+        fn = {"mx": bench_mx, "decode": bench_decode, "fp8": bench_fp8, "ragged_k": bench_ragged_k}[args.only]
+        print(json.dumps({args.only: fn(device, args.steps, args.warmup)}))
+        return
     T, E, k, d, f2 = 4096, 128, 4, 2880, 5760
     g = torch.Generator().manual_seed(2)
     x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)

@@ -272,6 +272,58 @@ constexpr int kTilePitch = 128 + 16;  // LDS bytes per column
 constexpr int kTileRows = 64 + 65 * 3;
 __device__ __forceinline__ int tile_row(int c) { return (c >> 2) + 65 * (c & 3); }
 
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Tiles are renumbered so that consecutive
+// tiles run on ONE XCD at about the same time, and the tiles of one column range are numbered consecutively along
+// the quantised axis: a column's quantised bytes (1440 per 2880 values of e2m1) are not a multiple of the 128-byte
+// line, so neighbouring tiles share the lines at their seams and the 64-byte pieces of the scale rows; in one L2
+// those are fetched (or written back) once, in two L2s twice.
+__device__ __forceinline__ int64_t tile_order(int64_t pid, int64_t total) {
+  const int64_t per = total / 8, extra = total % 8;
+  const int64_t grp = pid % 8, local = pid / 8;
+  return grp * per + (grp < extra ? grp : extra) + local;
+}
+
+typedef __attribute__((ext_vector_type(2))) unsigned short u16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+// two 16-bit floats (low half first) / scale -> two e2m1 codes in byte `SEL` of `old` (first value in the low nibble)
+template <int SRC>
+__device__ __forceinline__ uint32_t cvt_pk_fp4(uint32_t old, uint32_t pair, float scale, int sel) {
+  if constexpr (SRC == TK_BF16) {
+    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, pair);
+    return sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, v, scale, 0)
+           : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, v, scale, 1)
+           : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, v, scale, 2)
+                      : __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(old, v, scale, 3);
+  } else {
+    const half2_t v = __builtin_bit_cast(half2_t, pair);
+    return sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, v, scale, 0)
+           : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, v, scale, 1)
+           : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, v, scale, 2)
+                      : __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(old, v, scale, 3);
+  }
+}
+
+// byte pair `SEL` of `w` (two e2m1 codes, low nibble first) * scale -> two 16-bit floats (first value in the low half)
+template <int DST>
+__device__ __forceinline__ uint32_t cvt_pk_from_fp4(uint32_t w, float scale, int sel) {
+  if constexpr (DST == TK_BF16) {
+    const bf16x2_t r = sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0)
+                       : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1)
+                       : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2)
+                                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3);
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    const f16x2_t r = sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 0)
+                      : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 1)
+                      : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2)
+                                 : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3);
+    return __builtin_bit_cast(uint32_t, r);
+  }
+}
+
 template <int KIND>
 struct TileGeom {
   static constexpr int BB = KIND == TK_E2M1 ? 16 : 32;  // value bytes per block and column
@@ -322,11 +374,11 @@ __global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restr
   constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
   __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
   __shared__ uint8_t sc_s[kTileCols * NB];
-  int64_t bid = blockIdx.x;
-  const int64_t ct = bid % col_tiles;
-  bid /= col_tiles;
+  int64_t bid = tile_order(blockIdx.x, gridDim.x);
   const int64_t bt = bid % blk_tiles;
-  const int64_t o = bid / blk_tiles;
+  bid /= blk_tiles;
+  const int64_t ct = bid % col_tiles;
+  const int64_t o = bid / col_tiles;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
   const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
   const int c4 = lane * 4;  // this lane's four columns inside the tile
@@ -345,14 +397,47 @@ __global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restr
       const uint16_t e = (uint16_t)((c & 1) ? (w >> 16) : (w & 0xFFFFu));
       return Elem<SRC>::load(&e);
     };
+    // e2m1: the block maxima come from the 16-bit patterns themselves (|x| orders like its bits without the sign, two
+    // elements per instruction) and the hardware converts two 16-bit floats to two e2m1 codes while dividing by the
+    // power-of-two scale (round to nearest even, saturating at +-6, exact), so a pair of rows costs one byte permute
+    // and one conversion.  Blocks that hold an infinity or a NaN, or whose scale is so extreme that subnormal inputs
+    // could matter, take the fp32 path below.
+    uint32_t max01 = 0, max23 = 0;
+    if constexpr (KIND == TK_E2M1) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        max01 = pk_max_u16(max01, raw[i].x & 0x7FFF7FFFu);
+        max23 = pk_max_u16(max23, raw[i].y & 0x7FFF7FFFu);
+      }
+    }
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
+      uint4* dst = reinterpret_cast<uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
+      if constexpr (KIND == TK_E2M1) {
+        const uint32_t mx = c < 2 ? max01 : max23;
+        const uint32_t m16 = (c & 1) ? (mx >> 16) : (mx & 0xFFFFu);
+        const float mf = SRC == TK_BF16 ? hd_bits_f32(m16 << 16) : f16_bits_to_f32((uint16_t)m16);
+        const uint32_t sb = mx_scale_bits(mf, KIND, rounding);
+        const bool finite = SRC == TK_BF16 ? m16 < 0x7F80u : m16 < 0x7C00u;
+        if (finite && sb >= (16u << 23) && sb <= (250u << 23)) {
+          const float scale = hd_bits_f32(sb);
+          uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < 32; i += 2) {
+            const uint32_t lo = c < 2 ? raw[i].x : raw[i].y, hi = c < 2 ? raw[i + 1].x : raw[i + 1].y;
+            const uint32_t pair = __builtin_amdgcn_perm(hi, lo, (c & 1) ? 0x07060302u : 0x05040100u);  // (row i, row i+1) of column c
+            w[i >> 3] = cvt_pk_fp4<SRC>(w[i >> 3], pair, scale, (i >> 1) & 3);
+          }
+          dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+          sc_s[(c4 + c) * NB + b] = (uint8_t)(sb >> 23);
+          continue;
+        }
+      }
       float m = 0.0f;
 #pragma unroll
       for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(elem(i, c)));
       const uint32_t sbits = mx_scale_bits(m, KIND, rounding);
       const float inv = mx_inv_scale(sbits);
-      uint4* dst = reinterpret_cast<uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
       if (KIND == TK_E2M1) {
         // hardware conversion (round to nearest even, saturating at +-6); NaN is first turned into the infinity of
         // its sign so that it saturates like the reference's bit algorithm (mxfp.py:298-327)
@@ -389,11 +474,11 @@ __global__ __launch_bounds__(kThreads) void mx_up_tile(const uint8_t* __restrict
   constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
   __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
   __shared__ uint8_t sc_s[kTileCols * NB];
-  int64_t bid = blockIdx.x;
-  const int64_t ct = bid % col_tiles;
-  bid /= col_tiles;
+  int64_t bid = tile_order(blockIdx.x, gridDim.x);
   const int64_t bt = bid % blk_tiles;
-  const int64_t o = bid / blk_tiles;
+  bid /= blk_tiles;
+  const int64_t ct = bid % col_tiles;
+  const int64_t o = bid / col_tiles;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
   const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
   const int c4 = lane * 4;
@@ -404,69 +489,83 @@ __global__ __launch_bounds__(kThreads) void mx_up_tile(const uint8_t* __restrict
   for (int pass = 0; pass < NB / 4; ++pass) {
     const int b = wave + 4 * pass;
     if (blk0 + b >= L / 32 || col0 + c4 >= inner) continue;
-    uint32_t hp[32][2];  // the lane's four columns of each row as two packed pairs
-    auto put = [&](int i, int c, uint32_t h16) __attribute__((always_inline)) {
-      if (c & 1)
-        hp[i][c >> 1] |= h16 << 16;
-      else
-        hp[i][c >> 1] = h16;
-    };
-    auto put_f = [&](int i, int c, float f) __attribute__((always_inline)) {
-      uint16_t e;
-      Elem<DST>::store(&e, f);
-      put(i, c, e);
-    };
+    uint16_t* q = out + o * ostride_outer + (blk0 + b) * 32 * ostride_axis + col0 + c4;
+    if constexpr (KIND == TK_E2M1) {
+      // Common case, all four blocks of the lane have a scale for which element * scale is a normal number of the
+      // target type whatever the element: the hardware conversion (two codes -> two scaled 16-bit floats, exact, no
+      // clamp needed) yields rows (i, i+1) of one column, a byte permute per output dword regroups two columns'
+      // results into (column c, column c+1) of one row, and every 8 rows are stored as soon as they are complete.
+      uint32_t sb4[4];
+      bool all_fast = true;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t sb = sc_s[(c4 + c) * NB + b];
-      const uint4* srcp = reinterpret_cast<const uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
-      if (KIND == TK_E2M1) {
-        const uint4 w4 = srcp[0];
-        const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
-        // Hardware conversion where element * scale is a normal number of the target type whatever the element
-        // (then it is exact and needs no clamp); blocks with extreme scales take the bit algorithm.
-        const bool fast = DST == TK_BF16 ? (sb >= 8 && sb <= 248) : (sb >= 114 && sb <= 139);
-        if (fast) {
-          const float scale = hd_bits_f32(sb << 23);
+      for (int c = 0; c < 4; ++c) {
+        sb4[c] = sc_s[(c4 + c) * NB + b];
+        all_fast = all_fast && (DST == TK_BF16 ? (sb4[c] >= 8 && sb4[c] <= 248) : (sb4[c] >= 114 && sb4[c] <= 139));
+      }
+      if (all_fast) {
+        uint4 w4[4];
 #pragma unroll
-          for (int d = 0; d < 4; ++d) {
+        for (int c = 0; c < 4; ++c) w4[c] = *reinterpret_cast<const uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              uint32_t pr;
-              if (DST == TK_BF16) {
-                bf16x2_t r = g == 0   ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 0)
-                             : g == 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 1)
-                             : g == 2 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 2)
-                                      : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], scale, 3);
-                pr = __builtin_bit_cast(uint32_t, r);
-              } else {
-                f16x2_t r = g == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 0)
-                            : g == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 1)
-                            : g == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 2)
-                                     : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[d], scale, 3);
-                pr = __builtin_bit_cast(uint32_t, r);
-              }
-              put(d * 8 + g * 2, c, pr & 0xFFFFu);
-              put(d * 8 + g * 2 + 1, c, pr >> 16);
-            }
+        for (int d = 0; d < 4; ++d) {
+          uint32_t pr[4][4];  // [column][row pair of this group of 8 rows]
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const uint32_t w = d == 0 ? w4[c].x : d == 1 ? w4[c].y : d == 2 ? w4[c].z : w4[c].w;
+            const float scale = hd_bits_f32(sb4[c] << 23);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) pr[c][g] = cvt_pk_from_fp4<DST>(w, scale, g);
           }
-        } else {
 #pragma unroll
-          for (int i = 0; i < 32; ++i)
-            put_f(i, c, mx_dequant(bf16_bits_to_f32((uint16_t)e2m1_to_bf16_bits((w[i >> 3] >> (4 * (i & 7))) & 0xFu)), sb, mf, false));
+          for (int g = 0; g < 4; ++g) {
+            const int i = d * 8 + g * 2;
+            *reinterpret_cast<uint2*>(q + i * ostride_axis) =
+                make_uint2(__builtin_amdgcn_perm(pr[1][g], pr[0][g], 0x05040100u), __builtin_amdgcn_perm(pr[3][g], pr[2][g], 0x05040100u));
+            *reinterpret_cast<uint2*>(q + (i + 1) * ostride_axis) =
+                make_uint2(__builtin_amdgcn_perm(pr[1][g], pr[0][g], 0x07060302u), __builtin_amdgcn_perm(pr[3][g], pr[2][g], 0x07060302u));
+          }
         }
-      } else {
-        const uint4 a = srcp[0], bq = srcp[BB / 32];
-        const uint32_t w[8] = {a.x, a.y, a.z, a.w, bq.x, bq.y, bq.z, bq.w};
-#pragma unroll
-        for (int i = 0; i < 32; ++i)
-          put_f(i, c, mx_dequant(elem_f32<KIND>((w[i >> 2] >> (8 * (i & 3))) & 0xFFu), sb, mf, KIND == TK_E5M2));
+        continue;
       }
     }
-    uint16_t* q = out + o * ostride_outer + (blk0 + b) * 32 * ostride_axis + col0 + c4;
+    // general path (fp8 values, or a block with an extreme scale): element by element with the clamp, eight rows at a
+    // time so that only those rows' results are held in registers
+    uint4 wa[4], wb[4];
+    uint32_t sb4g[4];
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      *reinterpret_cast<uint2*>(q + i * ostride_axis) = make_uint2(hp[i][0], hp[i][1]);
+    for (int c = 0; c < 4; ++c) {
+      const uint4* srcp = reinterpret_cast<const uint4*>(vals_s + tile_row(c4 + c) * kTilePitch + b * BB);
+      wa[c] = srcp[0];
+      wb[c] = KIND == TK_E2M1 ? wa[c] : srcp[BB / 32];
+      sb4g[c] = sc_s[(c4 + c) * NB + b];
+    }
+    auto word = [](const uint4& v, int k) __attribute__((always_inline)) { return k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w; };
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      uint32_t hp[8][2];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          float f;
+          if (KIND == TK_E2M1) {
+            const uint32_t code = (word(wa[c], d) >> (4 * r)) & 0xFu;
+            f = mx_dequant(bf16_bits_to_f32((uint16_t)e2m1_to_bf16_bits(code)), sb4g[c], mf, false);
+          } else {
+            const int k = 2 * d + (r >> 2);  // dword of the block's 32 bytes
+            const uint32_t byte = (word(k < 4 ? wa[c] : wb[c], k & 3) >> (8 * (r & 3))) & 0xFFu;
+            f = mx_dequant(elem_f32<KIND>(byte), sb4g[c], mf, KIND == TK_E5M2);
+          }
+          uint16_t e;
+          Elem<DST>::store(&e, f);
+          if (c & 1)
+            hp[r][c >> 1] |= (uint32_t)e << 16;
+          else
+            hp[r][c >> 1] = e;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 8; ++r) *reinterpret_cast<uint2*>(q + (d * 8 + r) * ostride_axis) = make_uint2(hp[r][0], hp[r][1]);
     }
   }
 }
