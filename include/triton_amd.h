@@ -353,6 +353,9 @@ typedef struct tk_ragged_k_desc {
   const int32_t* slice_sizes;  /* [n_slices] reduction length per slice */
   const int32_t* a_slice_offs; /* [n_slices] first k of the slice in a */
   const int32_t* b_slice_offs; /* [n_slices] first k of the slice in b */
+  /* extent of the reduction dimension of a and of b (a is [M, a_k_extent], b is [b_k_extent, N]); every slice lies
+   * inside.  0 = not stated: the kernel then cannot bound its loads by the tensors' ends and takes its general path. */
+  int64_t a_k_extent, b_k_extent;
 } tk_ragged_k_desc;
 
 int32_t tk_ragged_k_gemm(const tk_ragged_k_desc* desc, tk_stream_t stream);

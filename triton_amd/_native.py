@@ -76,7 +76,7 @@ class RaggedKDesc(_c.Structure):
         ("b", _ptr), ("b_stride_k", _i64), ("b_stride_n", _i64),
         ("y", _ptr), ("y_dtype", _i32), ("y_stride_e", _i64), ("y_stride_m", _i64),
         ("M", _i32), ("N", _i32), ("n_slices", _i32),
-        ("slice_sizes", _ptr), ("a_slice_offs", _ptr), ("b_slice_offs", _ptr),
+        ("slice_sizes", _ptr), ("a_slice_offs", _ptr), ("b_slice_offs", _ptr), ("a_k_extent", _i64), ("b_k_extent", _i64),
     ]
 
 

@@ -271,6 +271,7 @@ def _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_in
     d.y, d.y_dtype = c.data_ptr(), nt.TORCH_TO_TK[out_dtype]
     d.y_stride_e, d.y_stride_m = c.stride(0), c.stride(1)
     d.M, d.N, d.n_slices = M, N, n_slices
+    d.a_k_extent, d.b_k_extent = a.shape[1], b.shape[0]
     sizes, a_offs, b_offs = b_ragged_metadata.slice_sizes, a_ragged_metadata.slice_offs, b_ragged_metadata.slice_offs
     assert sizes.dtype == a_offs.dtype == b_offs.dtype == torch.int32
     assert sizes.is_contiguous() and a_offs.is_contiguous() and b_offs.is_contiguous()
