@@ -1278,75 +1278,111 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
 // sc0 sc1 cache policy (write-through to memory / read from memory) and the counter is a device-scope atomic; the
 // alternative, a device-scope release fence per wave, writes back and invalidates a whole L2 each time and more than
 // doubled the kernel's time.  acc[g][j][i]: sub-fragment g (columns F*32 + g*16 + kg*4 + i), row fragment j.
-template <int MR>
-__device__ __forceinline__ void combine_epilogue(const GemmParams& p, f32x4_t (&acc)[2][MR], int expert, int off_m, int start_m, int eM, int F,
-                                                 int nfr, int lr, int kg) {
-  constexpr int kThrough = 1 | 16;  // aux bits of the buffer instructions: sc0 | sc1
-  const int N = p.N, k = p.combine_k;
-  const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
-  const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
-  float b4[2][4];
+// Operands of the combine epilogue that do not depend on the accumulators; the kernel fetches them before its K loop
+// so that their latency is not part of every wave's tail.
+template <int MR, int NFD>
+struct CombineOperands {
+  float gam[MR];
+  int dst[MR];          // destination row (flat position t * k + j) or -1
+  float b4[NFD][2][4];  // bias of the lane's columns
+};
+
+template <int MR, int NFD>
+__device__ __forceinline__ CombineOperands<MR, NFD> load_combine_operands(const GemmParams& p, int expert, int off_m, int start_m, int eM,
+                                                                          const int (&F)[NFD], int lr, int kg) {
+  CombineOperands<MR, NFD> o;
+  const int N = p.N;
 #pragma unroll
-  for (int g = 0; g < 2; ++g)
+  for (int fd = 0; fd < NFD; ++fd)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = F * 32 + g * 16 + kg * 4 + i;
-      b4[g][i] = (p.bias && n < N) ? load_scalar(p.bias, (int64_t)expert * p.bias_stride_e + n, p.bias_is_f32) : 0.f;
-    }
-  int token[MR];
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = F[fd] * 32 + g * 16 + kg * 4 + i;
+        o.b4[fd][g][i] = (p.bias && n < N) ? load_scalar(p.bias, (int64_t)expert * p.bias_stride_e + n, p.bias_is_f32) : 0.f;
+      }
 #pragma unroll
   for (int j = 0; j < MR; ++j) {
     const int row = off_m + j * 16 + lr;
     const bool ok = row < eM;
     const int srow = start_m + (ok ? row : eM - 1);
-    const float gam = p.gammas ? load_scalar(p.gammas, srow, p.gammas_is_f32) : 1.0f;
-    int dst = srow < p.scatter_len ? p.scatter[srow] : -1;
-    dst = ok ? dst : -1;
-    token[j] = dst >= 0 ? dst / k : -1;
-#pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      const int n0 = F * 32 + g * 16 + kg * 4;
-      const u32x2_t w = {pack_bf16x2((acc[g][j][0] + b4[g][0]) * gam, (acc[g][j][1] + b4[g][1]) * gam),
-                         pack_bf16x2((acc[g][j][2] + b4[g][2]) * gam, (acc[g][j][3] + b4[g][3]) * gam)};
-      const uint32_t off = (dst >= 0 && n0 < N) ? (uint32_t)dst * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
-      __builtin_amdgcn_raw_buffer_store_b64(w, yrsrc, off, 0, kThrough);
-    }
+    o.gam[j] = p.gammas ? load_scalar(p.gammas, srow, p.gammas_is_f32) : 1.0f;
+    const int dst = srow < p.scatter_len ? p.scatter[srow] : -1;
+    o.dst[j] = ok ? dst : -1;
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows have reached memory before it is counted
+  return o;
+}
+
+// The NFD fragments of a wave go through every step together (all stores, one wait, all counters, all loads), so the
+// chain of memory round trips at the end of a wave is as long for two fragments as for one.
+template <int MR, int NFD>
+__device__ __forceinline__ void combine_epilogue(const GemmParams& p, f32x4_t (&acc)[NFD][2][MR], const CombineOperands<MR, NFD>& o,
+                                                 const int (&F)[NFD], const bool (&live_f)[NFD], int nfr, int lr, int kg) {
+  constexpr int kThrough = 1 | 16;  // aux bits of the buffer instructions: sc0 | sc1
+  const int N = p.N, k = p.combine_k;
+  const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
+  const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
+  int token[MR];
 #pragma unroll
   for (int j = 0; j < MR; ++j) {
-    int seen = -1;
-    if (kg == 0 && token[j] >= 0)
-      seen = __hip_atomic_fetch_add(&p.combine_counters[(int64_t)token[j] * nfr + F], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    seen = __shfl(seen, lr);  // the row's four lanes (lr, lr + 16, ...) share lane lr's count
-    const bool last = token[j] >= 0 && seen == k - 1;
-    // (the loads below depend on the atomic's result, so they cannot be issued before it has been performed)
-    const uint32_t base = last ? (uint32_t)(token[j] * k) * row_bytes : kDroppedStore;
+    const int dst = o.dst[j];
+    const float gam = o.gam[j];
+    token[j] = dst >= 0 ? dst / k : -1;
 #pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      const int n0 = F * 32 + g * 16 + kg * 4;
-      float sum[4] = {0.f, 0.f, 0.f, 0.f};
-      for (int jj = 0; jj < k; ++jj) {
-        const uint32_t off = (last && n0 < N) ? base + (uint32_t)jj * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
-        const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(yrsrc, off, 0, kThrough);  // out-of-range lanes read zero
-        sum[0] += bits_f32(v.x << 16);
-        sum[1] += bits_f32(v.x & 0xFFFF0000u);
-        sum[2] += bits_f32(v.y << 16);
-        sum[3] += bits_f32(v.y & 0xFFFF0000u);
+    for (int fd = 0; fd < NFD; ++fd)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const int n0 = F[fd] * 32 + g * 16 + kg * 4;
+        const u32x2_t w = {pack_bf16x2((acc[fd][g][j][0] + o.b4[fd][g][0]) * gam, (acc[fd][g][j][1] + o.b4[fd][g][1]) * gam),
+                           pack_bf16x2((acc[fd][g][j][2] + o.b4[fd][g][2]) * gam, (acc[fd][g][j][3] + o.b4[fd][g][3]) * gam)};
+        const uint32_t off = (live_f[fd] && dst >= 0 && n0 < N) ? (uint32_t)dst * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
+        __builtin_amdgcn_raw_buffer_store_b64(w, yrsrc, off, 0, kThrough);
       }
-      if (last && n0 < N) {
-        uint16_t* o = p.combine_out + (int64_t)token[j] * p.combine_stride + n0;
-        if (n0 + 4 <= N && (p.combine_stride & 3) == 0) {
-          *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]));
-        } else {
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows have reached memory before it is counted
+  bool last[MR][NFD];
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (n0 + i < N) o[i] = f32_to_bf16_bits(sum[i]);
+  for (int j = 0; j < MR; ++j)
+#pragma unroll
+    for (int fd = 0; fd < NFD; ++fd) {
+      int seen = -1;
+      if (kg == 0 && token[j] >= 0 && live_f[fd])
+        seen = __hip_atomic_fetch_add(&p.combine_counters[(int64_t)token[j] * nfr + F[fd]], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      seen = __shfl(seen, lr);  // the row's four lanes (lr, lr + 16, ...) share lane lr's count
+      last[j][fd] = token[j] >= 0 && live_f[fd] && seen == k - 1;
+    }
+  // (the loads below depend on the atomics' results, so they cannot be issued before those have been performed)
+#pragma unroll
+  for (int j = 0; j < MR; ++j)
+#pragma unroll
+    for (int fd = 0; fd < NFD; ++fd) {
+      const uint32_t base = last[j][fd] ? (uint32_t)(token[j] * k) * row_bytes : kDroppedStore;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const int n0 = F[fd] * 32 + g * 16 + kg * 4;
+        float sum[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int jj = 0; jj < k; ++jj) {
+          const uint32_t off = (last[j][fd] && n0 < N) ? base + (uint32_t)jj * row_bytes + (uint32_t)n0 * 2u : kDroppedStore;
+          const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(yrsrc, off, 0, kThrough);  // out-of-range lanes read zero
+          sum[0] += bits_f32(v.x << 16);
+          sum[1] += bits_f32(v.x & 0xFFFF0000u);
+          sum[2] += bits_f32(v.y << 16);
+          sum[3] += bits_f32(v.y & 0xFFFF0000u);
+        }
+        if (last[j][fd] && n0 < N) {
+          uint16_t* out = p.combine_out + (int64_t)token[j] * p.combine_stride + n0;
+          if (n0 + 4 <= N && (p.combine_stride & 3) == 0) {
+            *reinterpret_cast<uint2*>(out) = make_uint2(pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]));
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (n0 + i < N) out[i] = f32_to_bf16_bits(sum[i]);
+          }
         }
       }
+      if (last[j][fd] && kg == 0)
+        __hip_atomic_store(&p.combine_counters[(int64_t)token[j] * nfr + F[fd]], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (last && kg == 0) __hip_atomic_store(&p.combine_counters[(int64_t)token[j] * nfr + F], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
 }
 
 template <int MR, int NFD, bool SWIGLU>
@@ -1374,8 +1410,13 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   const int ksplit = frag_tiles <= 1024 ? 4 : (frag_tiles <= 2048 ? 2 : 1);
   const int fpw = 4 / ksplit;                        // fragment groups per workgroup
   const int grid_n = (nslot + fpw - 1) / fpw;        // workgroups per row block
-  if ((int)blockIdx.x >= nblk * grid_n) return;
-  const int pid_n = blockIdx.x % grid_n, pid_m = blockIdx.x / grid_n;
+  // Workgroups go round-robin to the 8 XCDs.  With the row blocks a multiple of 8 workgroups apart, the workgroups that
+  // read one weight fragment for the different row blocks of an expert (an expert with more rows than a block holds)
+  // land on ONE XCD, close together in time, and share the fragment through its L2 instead of fetching it again.
+  const int grid_n8 = (grid_n + 7) & ~7;
+  if ((int)blockIdx.x >= nblk * grid_n8) return;
+  const int pid_n = blockIdx.x % grid_n8, pid_m = blockIdx.x / grid_n8;
+  if (pid_n >= grid_n) return;
   const int kslice = wave % ksplit;
   int expert, off_m, start_m, eM;
   if (p.slice_sizes) {
@@ -1490,6 +1531,12 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     }
   };
 
+  CombineOperands<MR, NFD> cops;
+  bool combine = false;
+  if constexpr (!SWIGLU) {
+    combine = p.combine_k > 0;
+    if (combine && live_wave && kslice == 0) cops = load_combine_operands<MR, NFD>(p, expert, off_m, start_m, eM, F, lr, kg);
+  }
   if (live_wave) {
     // prologue: fill the rings in the order the steady state leaves them (weights run WDD-1 stages ahead,
     // activations XDD-1)
@@ -1539,15 +1586,15 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[fd][g][j][i] += red[wave + o - 1][((fd * 2 + g) * MR + j) * 4 + i][lane];
   }
+  if constexpr (!SWIGLU) {
+    if (combine) {
+      if (live_wave) combine_epilogue<MR, NFD>(p, acc, cops, F, live_f, nfr, lr, kg);
+      return;
+    }
+  }
 #pragma unroll
   for (int fd = 0; fd < NFD; ++fd) {
     if (!live_f[fd]) continue;
-    if constexpr (!SWIGLU) {
-      if (p.combine_k > 0) {
-        combine_epilogue<MR>(p, acc[fd], expert, off_m, start_m, eM, F[fd], nfr, lr, kg);
-        continue;
-      }
-    }
     gemm_epilogue<16, 1, MR, 2, SWIGLU>(p, acc[fd], expert, off_m, start_m, eM, F[fd] * 32, F[fd] * 32 + 32 <= N, 0, lr, kg);
   }
 }
@@ -2220,7 +2267,7 @@ int32_t launch_mxd_n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t s
   GemmParams q = p;
   q.total_tiles = grid_m;  // row blocks in the non-ragged case
   // sized for a K-split of 4 (one fragment group per workgroup); with a smaller split the surplus leaves at once
-  const int64_t grid = (int64_t)grid_m * cdiv(cdiv(p.N, 32), NFD);
+  const int64_t grid = (int64_t)grid_m * ((cdiv(cdiv(p.N, 32), NFD) + 7) & ~int64_t(7));
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   if (swiglu)
