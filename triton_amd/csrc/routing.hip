@@ -37,10 +37,14 @@ __device__ inline float key_to_float(uint32_t k) {
 }
 
 // Orders this wave's LDS accesses: lanes exchange data through LDS without a workgroup barrier.
+// LDS instructions of one wave are executed in program order, so a lane's read that follows another lane's write in
+// the instruction stream sees it without any wait; all that is needed is that the compiler keeps the order.  (A
+// wavefront-scope fence does that too but also waits for the wave's outstanding GLOBAL stores, the results of the row
+// it has just finished: a full memory latency per row for nothing.)
 __device__ __forceinline__ void wave_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  asm volatile("" ::: "memory");
   __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  asm volatile("" ::: "memory");
 }
 
 // Wave-wide reductions with DPP lane exchanges (no LDS round trips): xor-1 and xor-2 inside a quad, mirror inside 8
@@ -146,7 +150,10 @@ struct TopkParams {
   int32_t* fill_c;
 };
 
-template <int DT, int EPL>
+// PROVIDED = the caller supplies the expert indices (p.use_provided_indx); as a template parameter so that the selecting
+// variant has no load inside its row loop: with one on some path the compiler waits for ALL outstanding memory
+// operations at the joins, i.e. for the previous row's stores.
+template <int DT, int EPL, bool PROVIDED>
 __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParams p) {
   __shared__ int32_t hist_s[kWaves][EPL * 64];
   __shared__ uint32_t words_s[kWaves][EPL * 2];
@@ -167,20 +174,31 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
       if (p.fill_c) p.fill_c[f] = -1;
     }
   }
-  // the next row's logits are fetched while the current row is being selected
-  float next_v[EPL];
-  if (!p.use_provided_indx && row_begin < row_end && row_begin < n_rows) {
+  // The logits of up to kBatch rows are fetched together before the first of them is selected: a wave walks its rows
+  // one after the other, and with one row in flight at a time every row cost a full memory latency.
+  constexpr int kBatch = EPL <= 2 ? 8 : EPL <= 4 ? 4 : EPL <= 8 ? 2 : 1;
+  float batch_v[kBatch][EPL];
+  for (int row0 = row_begin; row0 < row_end; row0 += kBatch) {
+  if constexpr (!PROVIDED) {
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) {
-      const int e = lane + 64 * i;
-      next_v[i] = e < E ? load_logit<DT>(p.logits, (int64_t)row_begin * p.stride_m + e) : 0.f;
+    for (int r = 0; r < kBatch; ++r) {
+      const int row = row0 + r;
+      if (row < row_end && row < n_rows) {
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const int e = lane + 64 * i;
+          batch_v[r][i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
+        }
+      }
     }
   }
-  for (int row = row_begin; row < row_end; ++row) {
-    if (row >= n_rows) break;
+#pragma unroll
+  for (int r = 0; r < kBatch; ++r) {
+    const int row = row0 + r;
+    if (row >= row_end || row >= n_rows) break;
     float myval = 0.f;
     int myidx = -1;
-    if (p.use_provided_indx) {
+    if constexpr (PROVIDED) {
       if (lane < k) {
         myidx = p.indx[(int64_t)row * k + lane];
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
@@ -188,21 +206,14 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
     } else {
       uint32_t key[EPL];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(next_v[i]) : 0u;
-      if (row + 1 < row_end && row + 1 < n_rows) {
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) {
-          const int e = lane + 64 * i;
-          next_v[i] = e < E ? load_logit<DT>(p.logits, (int64_t)(row + 1) * p.stride_m + e) : 0.f;
-        }
-      }
+      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(batch_v[r][i]) : 0u;
       wave_topk<EPL>(key, k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
       // softmax over the k kept logits in fp32; the largest sits in lane 0
       float vmax = myval;
-      if (p.use_provided_indx) {
+      if constexpr (PROVIDED) {
         float m = lane < k ? myval : -INFINITY;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
@@ -216,18 +227,21 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
     }
     if (lane < k) {
       if (p.vals) store_val<DT>(p.vals, (int64_t)row * k + lane, outv);
-      if (!p.use_provided_indx) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
+      if constexpr (!PROVIDED) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
     }
     const bool live = lane < k && myidx >= 0 && myidx < E;
     if (p.partials && live) atomicAdd(&hist_s[wave][myidx], 1);
     if (p.bitmatrix) {
-      for (int w = lane; w < words; w += 64) words_s[wave][w] = 0u;
+      // (words <= 64: at most 2048 experts.  No loops here: the compiler drains all outstanding global stores in front
+      // of a loop that touches memory, which would cost every row a store latency.)
+      if (lane < words) words_s[wave][lane] = 0u;
       wave_sync();
       if (live) atomicOr(&words_s[wave][myidx >> 5], 1u << (myidx & 31));
       wave_sync();
-      for (int w = lane; w < words; w += 64) p.bitmatrix[(int64_t)w * p.bm_stride_w + row] = words_s[wave][w];
+      if (lane < words) p.bitmatrix[(int64_t)lane * p.bm_stride_w + row] = words_s[wave][lane];
       wave_sync();
     }
+  }
   }
   if (p.partials && row_begin < p.T) {
     wave_sync();
@@ -257,7 +271,9 @@ constexpr int kQuantities = 1 + kNumBlockSizes;  // rows, then row blocks of 16,
 // block offsets, so a slice with thousands of blocks costs no more than an empty one.
 constexpr int kLdsOffsExperts = 1024;  // up to this many slices the offsets are also kept in LDS
 
-__device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int E, int32_t* offs0, const RaggedOut r, bool want_ragged) {
+// Returns the LDS copy of the slice offsets ([E + 1], valid after the caller's next workgroup barrier) or null when E
+// is too large for it.
+__device__ __forceinline__ const int32_t* ragged_metadata(const int32_t* slice_sizes, int E, int32_t* offs0, const RaggedOut r, bool want_ragged) {
   // LDS copies: row 0 = slice offsets (read back by the single-launch router), rows 1.. = block offsets, which the
   // schedule's binary search reads (seven dependent reads per slot; from global memory they dominated the kernel)
   __shared__ int32_t offs_s[kQuantities][kLdsOffsExperts + 1];
@@ -327,7 +343,7 @@ __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int 
       for (int b = 0; b < kNumBlockSizes; ++b) r.block_offs[b * r.block_offs_stride + E] = carry[1 + b];
     }
   }
-  if (!want_ragged) return;
+  if (!want_ragged) return use_lds ? offs_s[0] : nullptr;
   __threadfence_block();
   __syncthreads();
 #pragma unroll
@@ -348,6 +364,7 @@ __device__ __forceinline__ void ragged_metadata(const int32_t* slice_sizes, int 
       sched[i] = val;
     }
   }
+  return use_lds ? offs_s[0] : nullptr;
 }
 
 // Exclusive prefix over the waves' histograms, per expert.  Threads are laid out [group][expert] so that a
@@ -361,7 +378,9 @@ __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* parti
   groups = groups < 1 ? 1 : (groups > 32 ? 32 : groups);
   groups = groups > units ? units : groups;
   const int per_group = (units + groups - 1) / groups;
-  constexpr int kChunk = 8;
+  // loads of a chunk are in flight together: the kernel is one workgroup walking `units` rows of the workspace, and its
+  // time is the number of dependent memory round trips (two passes x run length / kChunk)
+  constexpr int kChunk = 16;
   for (int e0 = 0; e0 < E; e0 += kScanThreads) {  // more than one trip only when E > 1024 (then groups == 1)
     const int e = e0 + (int)(threadIdx.x % (unsigned)(E < kScanThreads ? E : kScanThreads));
     const int g = (int)(threadIdx.x / (unsigned)(E < kScanThreads ? E : kScanThreads));
@@ -560,7 +579,7 @@ struct SmallParams {
   RaggedOut r;
 };
 
-template <int DT, int EPL>
+template <int DT, int EPL, bool PROVIDED>
 __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallParams q) {
   __shared__ int32_t eid_s[kSmallEntries];
   __shared__ uint32_t val_s[kSmallEntries];
@@ -577,19 +596,30 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
   __syncthreads();
   // ---- phase 1: top-k per row (wave w takes rows w, w + 16, ...); the next row's logits are fetched while the
   // current row is selected, so a wave pays the memory latency once ----
-  float nv[EPL];
-  auto load_row = [&](int row) __attribute__((always_inline)) {
+  // (rows in batches, all loads of a batch in flight together and none inside the per-row code: see route_topk_kernel)
+  constexpr int kBatch = EPL <= 2 ? 4 : EPL <= 8 ? 2 : 1;
+  float nv[kBatch][EPL];
+  for (int row0 = wave; row0 < T && row0 < n_rows; row0 += kScanWaves * kBatch) {
+  if constexpr (!PROVIDED) {
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) {
-      const int e = lane + 64 * i;
-      nv[i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
+    for (int r = 0; r < kBatch; ++r) {
+      const int row = row0 + r * kScanWaves;
+      if (row < T && row < n_rows) {
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const int e = lane + 64 * i;
+          nv[r][i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
+        }
+      }
     }
-  };
-  if (!p.use_provided_indx && wave < T && wave < n_rows) load_row(wave);
-  for (int row = wave; row < T && row < n_rows; row += kScanWaves) {
+  }
+#pragma unroll
+  for (int r = 0; r < kBatch; ++r) {
+    const int row = row0 + r * kScanWaves;
+    if (row >= T || row >= n_rows) break;
     float myval = 0.f;
     int myidx = -1;
-    if (p.use_provided_indx) {
+    if constexpr (PROVIDED) {
       if (lane < k) {
         myidx = p.indx[(int64_t)row * k + lane];
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
@@ -597,15 +627,13 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
     } else {
       uint32_t key[EPL];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(nv[i]) : 0u;
-      const int nrow = row + kScanWaves;
-      if (nrow < T && nrow < n_rows) load_row(nrow);
+      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(nv[r][i]) : 0u;
       wave_topk<EPL>(key, k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
       float vmax;
-      if (p.use_provided_indx) {
+      if constexpr (PROVIDED) {
         float m = lane < k ? myval : -INFINITY;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
@@ -620,7 +648,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
     const bool live = lane < k && myidx >= 0 && myidx < E;
     if (lane < k) {
       if (p.vals) store_val<DT>(p.vals, (int64_t)row * k + lane, outv);
-      if (!p.use_provided_indx) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
+      if constexpr (!PROVIDED) p.indx[(int64_t)row * k + lane] = (int16_t)myidx;
       eid_s[row * k + lane] = live ? myidx : -1;
       // the gate value as it is stored (bits of the logits dtype)
       uint32_t bits;
@@ -634,30 +662,35 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
     }
     if (live) atomicAdd(&hist_s[myidx], 1);
     if (p.bitmatrix) {
-      for (int w = lane; w < words; w += 64) words_s[wave][w] = 0u;
+      // (words <= 64: at most 2048 experts.  No loops here: the compiler drains all outstanding global stores in front
+      // of a loop that touches memory, which would cost every row a store latency.)
+      if (lane < words) words_s[wave][lane] = 0u;
       wave_sync();
       if (live) atomicOr(&words_s[wave][myidx >> 5], 1u << (myidx & 31));
       wave_sync();
-      for (int w = lane; w < words; w += 64) p.bitmatrix[(int64_t)w * p.bm_stride_w + row] = words_s[wave][w];
+      if (lane < words) p.bitmatrix[(int64_t)lane * p.bm_stride_w + row] = words_s[wave][lane];
       wave_sync();
     }
+  }
   }
   __syncthreads();
   if (!q.col_sum) return;  // top-k only
   // ---- phase 2: histogram out, offsets and ragged metadata ----
   for (int e = threadIdx.x; e < E; e += kScanThreads) q.col_sum[e] = hist_s[e];
-  ragged_metadata(hist_s, E, q.col_offs, q.r, q.want_ragged != 0);  // sizes straight from LDS
+  const int32_t* offs_l = ragged_metadata(hist_s, E, q.col_offs, q.r, q.want_ragged != 0);  // sizes straight from LDS
   __threadfence_block();
   __syncthreads();
-  // ---- phase 3: stable ranks and the permutations ----
-  int total = q.col_offs[E];
+  // ---- phase 3: stable ranks and the permutations (the offsets come from the LDS copy when there is one: reading
+  // back what this workgroup has just written to global memory costs a full memory round trip) ----
+  const int32_t* offs = offs_l ? offs_l : q.col_offs;
+  int total = offs[E];
   for (int f = threadIdx.x; f < R; f += kScanThreads) {
     const int e = eid_s[f];
     int pos = -1;
     if (e >= 0) {
       int rank = 0;
       for (int g = 0; g < f; ++g) rank += eid_s[g] == e ? 1 : 0;
-      pos = q.col_offs[e] + rank;
+      pos = offs[e] + rank;
       q.col_sorted[pos] = f;
       if (q.gather_out) q.gather_out[pos] = f / k;
       if (q.gammas_out) {
@@ -712,7 +745,11 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
     const int64_t f = f0 + lane;
     const bool in = f < f_end;
     int e = -1;
-    if (in && f < n_valid) e = p.indx16 ? (int)p.indx16[f] : p.indx32[f];
+    uint32_t gate_bits = 0;  // fetched together with the index: its latency is hidden behind the ranking below
+    if (in && f < n_valid) {
+      e = p.indx16 ? (int)p.indx16[f] : p.indx32[f];
+      if (p.gammas_out) gate_bits = p.vals_bytes == 4 ? static_cast<const uint32_t*>(p.vals)[f] : (uint32_t) static_cast<const uint16_t*>(p.vals)[f];
+    }
     const bool valid = e >= 0 && e < E;
     int pos = -1;
     unsigned long long todo = __ballot(valid);
@@ -732,9 +769,9 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
       if (p.gather_out) p.gather_out[pos] = (int32_t)(f / k);
       if (p.gammas_out) {
         if (p.vals_bytes == 4)
-          static_cast<uint32_t*>(p.gammas_out)[pos] = static_cast<const uint32_t*>(p.vals)[f];
+          static_cast<uint32_t*>(p.gammas_out)[pos] = gate_bits;
         else
-          static_cast<uint16_t*>(p.gammas_out)[pos] = static_cast<const uint16_t*>(p.vals)[f];
+          static_cast<uint16_t*>(p.gammas_out)[pos] = (uint16_t)gate_bits;
       }
     }
   }
@@ -755,7 +792,10 @@ int32_t launch_topk(const TopkParams& p, int units, hipStream_t st) {
   const int epl = (p.E + 63) / 64;
 #define TK_EPL(N)                                                                                              \
   if (epl <= N) {                                                                                              \
-    hipLaunchKernelGGL((route_topk_kernel<DT, N>), dim3(grid), dim3(kWaves * 64), 0, st, p);                    \
+    if (p.use_provided_indx)                                                                                   \
+      hipLaunchKernelGGL((route_topk_kernel<DT, N, true>), dim3(grid), dim3(kWaves * 64), 0, st, p);           \
+    else                                                                                                       \
+      hipLaunchKernelGGL((route_topk_kernel<DT, N, false>), dim3(grid), dim3(kWaves * 64), 0, st, p);          \
     return check_launch("route_topk_kernel");                                                                  \
   }
   TK_EPL(1)
@@ -773,7 +813,10 @@ int32_t launch_small_dt(const SmallParams& q, hipStream_t st) {
   const int epl = (q.t.E + 63) / 64;
 #define TK_EPL(N)                                                                                              \
   if (epl <= N) {                                                                                              \
-    hipLaunchKernelGGL((route_small_kernel<DT, N>), dim3(1), dim3(kScanThreads), 0, st, q);                     \
+    if (q.t.use_provided_indx)                                                                                 \
+      hipLaunchKernelGGL((route_small_kernel<DT, N, true>), dim3(1), dim3(kScanThreads), 0, st, q);            \
+    else                                                                                                       \
+      hipLaunchKernelGGL((route_small_kernel<DT, N, false>), dim3(1), dim3(kScanThreads), 0, st, q);           \
     return check_launch("route_small_kernel");                                                                 \
   }
   TK_EPL(1)
