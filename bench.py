@@ -332,7 +332,7 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
 
     ms = time_steps(step, steps, warmup)
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
-    # algorithmic bytes with one-byte activations: x_q + scales, W1, h_q twice, W2, y twice, out (SURVEY accounting)
+    # algorithmic bytes with one-byte activations: x_q + scales, W1, h_q twice, W2, y twice, out
     R = T * k
     E = W["b1"].shape[0]
     nbytes = (R * d * 33 / 32 + E * (d * f2 * 17 / 32 + f2 * 2) + 2 * R * (f2 // 2) * 33 / 32 + E * ((f2 // 2) * d * 17 / 32 + d * 2) + 2 * R * d * 2 + T * d * 2)
