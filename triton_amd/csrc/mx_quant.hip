@@ -284,6 +284,7 @@ __device__ __forceinline__ int64_t tile_order(int64_t pid, int64_t total) {
 }
 
 typedef __attribute__((ext_vector_type(2))) unsigned short u16x2_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
   return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
@@ -352,46 +353,38 @@ __device__ __forceinline__ void tile_move(uint8_t* vals_s, uint8_t* sc_s, uint8_
         *l = *g;
     }
   }
-#pragma unroll
-  for (int it = 0; it < NB; ++it) {
-    const int q = it * kThreads + threadIdx.x;
-    const int col = q / NB, b = q % NB;
-    if (col0 + col < inner && blk0 + b < nblk) {
+  // scales: a column's NB bytes are contiguous in both places, so one thread moves them in one piece (4 or 8 bytes at
+  // any alignment) unless the tile hangs over the end of the axis; single-byte accesses cost an instruction and a
+  // memory transaction each
+  static_assert(kTileCols == kThreads, "one column per thread");
+  {
+    const int col = threadIdx.x;
+    if (col0 + col < inner && blk0 < nblk) {
       const int64_t line = line_of(o, col0 + col, inner, inner_last);
-      if (TO_GLOBAL)
-        gscales[line * nblk + blk0 + b] = sc_s[col * NB + b];
-      else
-        sc_s[col * NB + b] = gscales[line * nblk + blk0 + b];
+      uint8_t* g = gscales + line * nblk + blk0;
+      uint8_t* l = sc_s + col * NB;
+      if (blk0 + NB <= nblk) {
+        if (TO_GLOBAL)
+          __builtin_memcpy(g, l, NB);
+        else
+          __builtin_memcpy(l, g, NB);
+      } else {
+        for (int b = 0; blk0 + b < nblk; ++b) {
+          if (TO_GLOBAL)
+            g[b] = l[b];
+          else
+            l[b] = g[b];
+        }
+      }
     }
   }
 }
 
+// Quantises the lane's 32 rows x 4 columns of block `b` (raw[i] = row i, two 16-bit elements per dword) into the
+// tile's LDS staging arrays.
 template <int SRC, int KIND>
-__global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restrict__ src, int64_t stride_outer, int64_t stride_axis,
-                                                         int64_t L, int64_t inner, int64_t inner_last, int64_t col_tiles,
-                                                         int64_t blk_tiles, uint8_t* __restrict__ out_vals,
-                                                         uint8_t* __restrict__ out_scales, int rounding) {
+__device__ __forceinline__ void quantise_block_to_lds(const uint2 (&raw)[32], uint8_t* vals_s, uint8_t* sc_s, int c4, int b, int rounding) {
   constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
-  __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
-  __shared__ uint8_t sc_s[kTileCols * NB];
-  int64_t bid = tile_order(blockIdx.x, gridDim.x);
-  const int64_t bt = bid % blk_tiles;
-  bid /= blk_tiles;
-  const int64_t ct = bid % col_tiles;
-  const int64_t o = bid / col_tiles;
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
-  const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
-  const int c4 = lane * 4;  // this lane's four columns inside the tile
-#pragma unroll 1
-  for (int pass = 0; pass < NB / 4; ++pass) {
-    const int b = wave + 4 * pass;
-    if (blk0 + b >= L / 32 || col0 + c4 >= inner) continue;
-    const uint16_t* p = src + o * stride_outer + (blk0 + b) * 32 * stride_axis + col0 + c4;
-    // the 32 rows stay packed (two 16-bit elements per register) and are widened where they are used: half the
-    // registers of an fp32 copy, which is what lets four workgroups share a CU and overlap their load phases
-    uint2 raw[32];
-#pragma unroll
-    for (int i = 0; i < 32; ++i) raw[i] = *reinterpret_cast<const uint2*>(p + i * stride_axis);
     auto elem = [&](int i, int c) __attribute__((always_inline)) {
       const uint32_t w = c < 2 ? raw[i].x : raw[i].y;
       const uint16_t e = (uint16_t)((c & 1) ? (w >> 16) : (w & 0xFFFFu));
@@ -462,6 +455,35 @@ __global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restr
       }
       sc_s[(c4 + c) * NB + b] = (uint8_t)(sbits >> 23);
     }
+}
+
+template <int SRC, int KIND>
+__global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restrict__ src, int64_t stride_outer, int64_t stride_axis,
+                                                         int64_t L, int64_t inner, int64_t inner_last, int64_t col_tiles,
+                                                         int64_t blk_tiles, uint8_t* __restrict__ out_vals,
+                                                         uint8_t* __restrict__ out_scales, int rounding) {
+  constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
+  __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
+  __shared__ uint8_t sc_s[kTileCols * NB];
+  int64_t bid = tile_order(blockIdx.x, gridDim.x);
+  const int64_t bt = bid % blk_tiles;
+  bid /= blk_tiles;
+  const int64_t ct = bid % col_tiles;
+  const int64_t o = bid / col_tiles;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
+  const int64_t col0 = ct * kTileCols, blk0 = bt * NB;
+  const int c4 = lane * 4;  // this lane's four columns inside the tile
+#pragma unroll 1
+  for (int pass = 0; pass < NB / 4; ++pass) {
+    const int b = wave + 4 * pass;
+    if (blk0 + b >= L / 32 || col0 + c4 >= inner) continue;
+    const uint16_t* p = src + o * stride_outer + (blk0 + b) * 32 * stride_axis + col0 + c4;
+    // the 32 rows stay packed (two 16-bit elements per register) and are widened where they are used: half the
+    // registers of an fp32 copy, which is what lets four workgroups share a CU and overlap their load phases
+    uint2 raw[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) raw[i] = *reinterpret_cast<const uint2*>(p + i * stride_axis);
+    quantise_block_to_lds<SRC, KIND>(raw, vals_s, sc_s, c4, b, rounding);
   }
   __syncthreads();
   tile_move<KIND, true>(vals_s, sc_s, out_vals, out_scales, o, col0, blk0, L, inner, inner_last);
