@@ -381,6 +381,68 @@ __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(int32_t* parti
   // loads of a chunk are in flight together: the kernel is one workgroup walking `units` rows of the workspace, and its
   // time is the number of dependent memory round trips (two passes x run length / kChunk)
   constexpr int kChunk = 16;
+  // Vector form (E a multiple of 4, the usual case): a thread owns FOUR experts of a run of units and moves them as one
+  // 16-byte piece, so 1024 threads cover E / 4 columns x up to 32 runs; a run of at most kVec units stays in registers
+  // between the two passes (one memory round trip to read, one to write), longer runs are walked in chunks of kVec.
+  constexpr int kVec = 12;
+  if (E % 4 == 0 && E / 4 <= kScanThreads && (reinterpret_cast<uintptr_t>(partials) & 15) == 0 && (reinterpret_cast<uintptr_t>(col_sum) & 15) == 0) {
+    __shared__ int4 run_total4[kScanThreads];
+    const int w4 = E / 4;
+    int vgroups = kScanThreads / w4;
+    vgroups = vgroups > 32 ? 32 : vgroups;
+    vgroups = vgroups > units ? units : vgroups;
+    vgroups = vgroups < 1 ? 1 : vgroups;
+    const int vper = (units + vgroups - 1) / vgroups;
+    const int e4 = (int)(threadIdx.x % (unsigned)w4), g = (int)(threadIdx.x / (unsigned)w4);
+    const bool active = g < vgroups;
+    const int u_begin = g * vper;
+    int u_end = u_begin + vper;
+    u_end = u_end < units ? u_end : units;
+    int4* p4 = reinterpret_cast<int4*>(partials);
+    const bool single = vper <= kVec;
+    int4 v[kVec];
+    int4 sum = make_int4(0, 0, 0, 0);
+    if (active) {
+      for (int u = u_begin; u < u_end; u += kVec) {
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) v[i] = u + i < u_end ? p4[(int64_t)(u + i) * w4 + e4] : make_int4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) {
+          sum.x += v[i].x;
+          sum.y += v[i].y;
+          sum.z += v[i].z;
+          sum.w += v[i].w;
+        }
+      }
+      run_total4[threadIdx.x] = sum;
+    }
+    __syncthreads();
+    if (active) {
+      int4 run = make_int4(0, 0, 0, 0);
+      for (int gg = 0; gg < g; ++gg) {
+        const int4 t = run_total4[gg * w4 + e4];
+        run.x += t.x;
+        run.y += t.y;
+        run.z += t.z;
+        run.w += t.w;
+      }
+      for (int u = u_begin; u < u_end; u += kVec) {
+        if (!single) {
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) v[i] = u + i < u_end ? p4[(int64_t)(u + i) * w4 + e4] : make_int4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) {
+          if (u + i < u_end) p4[(int64_t)(u + i) * w4 + e4] = run;
+          run.x += v[i].x;
+          run.y += v[i].y;
+          run.z += v[i].z;
+          run.w += v[i].w;
+        }
+      }
+      if (g == vgroups - 1) reinterpret_cast<int4*>(col_sum)[e4] = run;
+    }
+  } else
   for (int e0 = 0; e0 < E; e0 += kScanThreads) {  // more than one trip only when E > 1024 (then groups == 1)
     const int e = e0 + (int)(threadIdx.x % (unsigned)(E < kScanThreads ? E : kScanThreads));
     const int g = (int)(threadIdx.x / (unsigned)(E < kScanThreads ? E : kScanThreads));
@@ -777,12 +839,14 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
   }
 }
 
-// Rows one wave routes: one for small batches (latency), more as T grows so that the per-wave
-// histograms the scan has to walk stay at <= 512 rows of the workspace up to T = 8192 (<= 1024 beyond).
-int rows_per_wave_for(int T) {
+// Rows one wave routes: one for small batches (latency), more as T grows so that the per-wave histograms the scan has
+// to walk stay at <= 1024 rows of the workspace (<= 512 when a row is long: E > 256).  A wave pays about 1.2 us per row
+// (a dependent chain of lane exchanges, alone on its SIMD), the scan one memory round trip per 16 workspace rows of a
+// run, so shorter waves and a longer workspace are the better trade up to here.
+int rows_per_wave_for(int T, int E) {
+  const int64_t max_units = E <= 256 ? 1024 : 512;
   int rpw = 1;
-  while ((int64_t)rpw * 512 < T && rpw < 16) rpw *= 2;
-  while ((int64_t)rpw * 1024 < T) rpw *= 2;
+  while ((int64_t)rpw * max_units < T) rpw *= 2;
   return rpw;
 }
 
@@ -842,7 +906,7 @@ using namespace tk;
 
 extern "C" int64_t tk_route_workspace_bytes(int32_t T, int32_t E) {
   if (T <= 0 || E <= 0) return 0;
-  const int rpw = rows_per_wave_for(T);
+  const int rpw = rows_per_wave_for(T, E);
   const int64_t units = (T + rpw - 1) / rpw;
   const int64_t units_pad = (units + kWaves - 1) / kWaves * kWaves;
   return (units_pad * E + (int64_t)E + 1) * 4;
@@ -862,7 +926,7 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   if (want_meta && (!d->col_sorted_indx || !d->row_sorted_indx || !workspace)) return fail(TK_ERR_INVALID, "tk_route: metadata outputs / workspace missing");
   if (d->indx_dtype != TK_I16) return fail(TK_ERR_UNSUPPORTED, "tk_route: indx must be int16");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int rpw = rows_per_wave_for(T);
+  const int rpw = rows_per_wave_for(T, E);
   const int units = (T + rpw - 1) / rpw;
   const int units_pad = (units + kWaves - 1) / kWaves * kWaves;
   int32_t* partials = static_cast<int32_t*>(workspace);
