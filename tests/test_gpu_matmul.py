@@ -480,3 +480,61 @@ def test_mxfp8_activations_with_fused_mx_output(mods, device, swiglu, scatter, b
     assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
     # the quantised result is close to the unquantised GEMM (e4m3 has 3 mantissa bits: half a step is 2^-4 relative)
     assert_close(h, got, maxtol=1.0, rmstol=4e-2, what="MX output against the unquantised result")
+
+
+@pytest.mark.parametrize("kind", ["bf16", "mxfp4", "mxfp4_tiled"])
+@pytest.mark.parametrize("B, m, n, k", [(3, 200, 256, 256), (10, 72, 576, 768), (4, 1, 64, 128)])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_batched_matmul(mods, device, kind, B, m, n, k, swiglu):
+    """Batched mode (python/triton_kernels/tests/test_matmul.py:116-127,144-176 "batched"): a [B, m, k] x b [B, k, n] with a
+    bias per batch; against the oracle's ragged GEMM with B slices of m rows (what batched mode is), output [B, m, n_out]."""
+    mm, _, _ = mods
+    from triton_amd.swiglu import swiglu_fn
+    g = torch.Generator().manual_seed(B * 1000 + m + n + k)
+    a = torch.randn((B, m, k), generator=g).to(torch.bfloat16)
+    bias = torch.randn((B, n), generator=g)
+    w = _make_w(B, k, n, kind, g, device)
+    sizes = torch.full((B, ), m, dtype=torch.int32)
+    ref = omoe.matmul(a.reshape(B * m, k), w["w_cpu"], bias, sizes, w_mx_scale=w.get("scale_cpu"))
+    act = None
+    if swiglu:
+        act = mm.FusedActivation(mm.FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0))
+        ref = omoe.swiglu(ref, 1.702, 7.0)
+    pc = mm.PrecisionConfig(b_mx_scale=w.get("scale_dev"))
+    out = mm.matmul(a.to(device), w["w_dev"], bias.to(device), precision_config=pc, fused_activation=act)
+    assert out.shape == (B, m, n // (2 if swiglu else 1)) and out.dtype == torch.bfloat16
+    if swiglu:  # computed on the fp32 accumulators, the oracle rounds the GEMM output to bf16 first (see test_fused_swiglu)
+        assert_close(ref.reshape(out.shape), out, maxtol=3e-2, what="batched swiglu(y)")
+    else:
+        assert_allclose_gate(ref.reshape(out.shape), out, what="batched matmul")
+
+
+@pytest.mark.parametrize("kind", ["mxfp4_tiled", "fp8_tiled"])
+@pytest.mark.parametrize("sizes", [[200], [200, 200, 200], [130, 0, 300], [1, 1, 1, 1, 1, 1, 1]])
+def test_persistent_kernels_with_a_handful_of_tiles(mods, device, kind, sizes):
+    """The persistent prefill kernels launch one workgroup per tile when there are fewer tiles than compute units; with
+    fewer than 8 workgroups some XCD queue of the tile claimer has no workgroup of its own, and its tiles must still be
+    computed.  The output buffer is pre-filled with NaN so that a tile nobody wrote cannot pass."""
+    mm, _, tensor = mods
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import make_default_matmul_fp8_w_layout
+    g = torch.Generator().manual_seed(len(sizes) * 100 + sizes[0])
+    E, m, k, n = len(sizes), sum(sizes), 256, 256
+    st = torch.tensor(sizes, dtype=torch.int32)
+    md = tensor.make_ragged_tensor_metadata(st.to(device), m)
+    bias = torch.randn((E, n), generator=g)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
+    if kind == "mxfp4_tiled":
+        x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+        w = _make_w(E, k, n, kind, g, device)
+        y = mm.matmul(x.to(device), w["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=w["scale_dev"]), c=out)
+        ref = omoe.matmul(x, w["w_cpu"], bias, st, w_mx_scale=w["scale_cpu"])
+    else:
+        xq, sx, wq, sw = _fp8_operands(m, n, k, E, g)
+        wd = convert_layout(wrap_torch_tensor(wq.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)), make_default_matmul_fp8_w_layout())
+        pc = mm.PrecisionConfig(a_mx_tensor_scale=sx.to(device), b_mx_tensor_scale=sw.to(device), out_dtype=torch.bfloat16)
+        y = mm.matmul(xq.to(device), wd, bias.to(device), md, precision_config=pc, c=out)
+        ref = omoe.matmul(xq, wq, bias, st, x_row_scale=sx, w_col_scale=sw, out_dtype=torch.bfloat16)
+    assert y.data_ptr() == out.data_ptr()
+    assert not torch.isnan(y).any(), "rows that no tile wrote"
+    assert_allclose_gate(ref, y, what="few tiles")

@@ -902,7 +902,9 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   };
 
   // (with the same number of tiles for every workgroup the static schedule is already even, and measured faster)
-  const bool dyn = p.tile_counters != nullptr && live % grid != 0;
+  // (claiming also needs at least one workgroup per queue, i.e. a grid of 8 or more: a queue's tiles are reached
+  // through the workgroups that start on it)
+  const bool dyn = p.tile_counters != nullptr && live % grid != 0 && grid >= 8;
   TileClaimer claimer;
   int round0 = 0;
   int pid, pid_next;  // this workgroup's current and next tile id (-1 = none)
@@ -1636,7 +1638,9 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   const int live = p.slice_sizes ? p.block_offs[p.n_slices] * p.grid_n : p.total_tiles;
   __shared__ int next_tile_s[2];  // written by thread 0 before a tile's first barrier: the id of the tile after it
   int tile_par = 0, n_tile = 0;
-  const bool dyn = p.tile_counters != nullptr;
+  // (claiming needs at least one workgroup per XCD queue: a queue's tiles are reached through the workgroups that
+  // start on it)
+  const bool dyn = p.tile_counters != nullptr && gridDim.x >= 8;
   TileClaimer claimer;
   int pid = claimer.init(p.tile_counters, live), round0 = 0;
   // (dynamic: a workgroup whose queue is shorter than its first index gets no tile at all, which only happens when

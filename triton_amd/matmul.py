@@ -12,7 +12,7 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
     fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
 
 Options of the reference signature that this build rejects with NotImplementedError: `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
-output / accumulator scales, batched 3-D activations, split-k.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
+output / accumulator scales, split-k.  Batched 3-D activations run as a ragged problem with equal slices.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
 `flex_ctx.rhs_data.scale`) are folded into the per-row / per-column scales of the epilogue.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
 MX quantiser kernel on the same stream.
 """
@@ -219,6 +219,43 @@ def _localise_remapped_metadata(md: RaggedTensorMetadata, n_local: int, n_rows: 
     return RaggedTensorMetadata(sizes, md.slice_offs[:n_local + 1], local.block_offs_data, local.block_schedule_data)
 
 
+_BATCH_METADATA = {}
+
+
+def _matmul_batched(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, betas, gammas, out_alpha, c,
+                    fused_comm, fused_activation, epilogue, c_acc_in):
+    """Batched mode (triton_kernels/matmul.py:270-277): a [B, M, K] x b [B, K, N] -> [B, M, N], batch i with weight i.
+    It is the ragged problem with B slices of exactly M rows, so it runs on the ragged kernels with metadata built
+    once per (B, M) and kept; no gather, scatter or ragged metadata of the caller's own."""
+    assert gather_indx is None, "gather not supported in batched mode"
+    assert scatter_indx is None, "scatter not supported in batched mode"
+    assert a_ragged_metadata is None, "x cannot be ragged in batched mode"
+    assert fused_comm is None, "fused comm is not supported in batched mode"
+    b_data = b.storage.data if isinstance(b, Tensor) else b
+    assert len(b.shape) == 3 and b.shape[0] == a.shape[0], "batched mode needs one weight matrix per batch"
+    del b_data
+    B, M, K = a.shape
+    key = (B, M, str(a.device))
+    md = _BATCH_METADATA.get(key)
+    if md is None:
+        from .tensor import make_ragged_tensor_metadata
+        md = make_ragged_tensor_metadata(torch.full((B, ), M, dtype=torch.int32, device=a.device), B * M)
+        if len(_BATCH_METADATA) >= 16:
+            _BATCH_METADATA.pop(next(iter(_BATCH_METADATA)))
+        _BATCH_METADATA[key] = md
+    if gammas is not None:
+        gammas = gammas.repeat(B) if gammas.shape[0] == M else gammas
+    if bias is not None and bias.ndim == 1:
+        bias = bias[None].expand(B, -1)
+    c2 = None
+    if c is not None:
+        assert c.ndim == 3 and c.shape[0] == B and c.is_contiguous()
+        c2 = c.view(B * M, c.shape[-1])
+    y = matmul(a.reshape(B * M, K), b, bias, md, None, None, None, precision_config, betas, gammas, out_alpha, c2, None,
+               fused_activation, epilogue, c_acc_in)
+    return y.view(B, M, y.shape[-1]) if c is None else c
+
+
 def _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_indx, scatter_indx, precision_config, betas,
                      gammas, out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in):
     """The reduction dimension is ragged (triton_kernels/matmul.py:376-384): one [M, N] output per slice,
@@ -300,6 +337,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if b_ragged_metadata is not None:
         return _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_indx, scatter_indx, precision_config,
                                 betas, gammas, out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in)
+    a_data = a.storage.data if isinstance(a, Tensor) else a
+    if a_data.ndim == 3:
+        return _matmul_batched(a_data, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, betas, gammas,
+                               out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in)
     if c_acc_in is not None:
         raise NotImplementedError("c_acc_in is not supported")
     if fused_comm is not None:
@@ -347,8 +388,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if isinstance(a, Tensor):
         a = a.storage.data
     a = flex.lhs_data.reinterpret(a)
-    if a.ndim != 2:
-        raise NotImplementedError("batched 3-D activations are not supported")
+    assert a.ndim == 2
     nt.require_gpu(a, "a")
     # ---- weights -------------------------------------------------------------------------------
     b_scale = precision_config.b_mx_scale
