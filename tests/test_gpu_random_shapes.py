@@ -24,7 +24,7 @@ def _random_sizes(g, n_slices, total):
     return sizes.to(torch.int32)
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", list(range(40)) + [100 + i for i in range(9)])
 def test_random_ragged_problem(device, seed):
     import triton_amd.matmul as mm
     import triton_amd.tensor as tensor
@@ -40,6 +40,9 @@ def test_random_ragged_problem(device, seed):
     k = 32 * ri(4, 24)                       # 128 .. 768, not always a multiple of the K-stage
     swiglu = bool(ri(0, 1))
     n = (16 if swiglu else 8) * ri(2, 80)    # up to 640 (1280 with swiglu), rarely a multiple of the tile width
+    if seed >= 100:  # enough tiles for several rounds of the persistent grids (256 workgroups), around their multiples
+        E, m, k = ri(8, 40), ri(12000, 40000), 32 * ri(4, 12)
+        n = (16 if swiglu else 8) * ri(100, 200)
     do_gather, do_scatter, do_gamma = bool(ri(0, 1)), bool(ri(0, 1)), bool(ri(0, 1))
     sizes = _random_sizes(g, E, m)
     md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
