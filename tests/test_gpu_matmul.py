@@ -116,6 +116,49 @@ def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatt
     assert_allclose_gate(ref, got, what="y")
 
 
+@pytest.mark.parametrize("m, n, k, mode", [(16, 256, 256, "ragged"), (300, 400, 416, "ragged"), (1000, 704, 832, "ragged"),
+                                           (600, 400, 416, "plain"), (5, 2880, 2880, "ragged")])
+@pytest.mark.parametrize("block_m", [16, 32, 64, 128])
+@pytest.mark.parametrize("k_major", [False, True])
+@pytest.mark.parametrize("do_gather, do_scatter, do_gamma, swiglu", [(False, False, False, False), (True, False, False, True),
+                                                                     (False, True, True, False), (True, True, False, False)])
+def test_matmul_fp16(mods, device, m, n, k, mode, block_m, k_major, do_gather, do_scatter, do_gamma, swiglu):
+    """fp16 x fp16 -> fp16 (the reference's test_matmul.py float16 cases): the bf16 kernel with the fp16 MFMA and an
+    fp16 epilogue."""
+    mm, sw, tensor = mods
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + k + block_m + 17 * k_major)
+    n_slices = 10 if mode == "ragged" else 1
+    x = torch.randn((m, k), generator=g).to(torch.float16)
+    w = (torch.randn((n_slices, k, n), generator=g) * 2 / k**0.5).to(torch.float16)
+    wd = w.to(device)
+    if k_major:
+        wd = wd.transpose(-1, -2).contiguous().transpose(-1, -2)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g) if mode == "ragged" else None
+    gather = torch.randint(0, m, (m, ), generator=g, dtype=torch.int32) if do_gather else None
+    scatter = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    gammas = 2.0**torch.randint(-5, 0, (m, ), generator=g).float() if do_gamma else None
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m) if sizes is not None else None
+    dev = lambda t: None if t is None else t.to(device)
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    kw = dict(fused_activation=act) if swiglu else {}
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(x.to(device), wd, dev(bias) if mode == "ragged" else dev(bias[0]), md, gather_indx=dev(gather),
+                      scatter_indx=dev(scatter), gammas=dev(gammas), **kw)
+    assert y.dtype == torch.float16
+    if swiglu:
+        h = omoe.matmul(x, w, bias, sizes, gather_indx=gather, out_dtype=torch.float32)
+        ref = omoe.swiglu(h, 1.702, 7.0, out_dtype=torch.float32)
+        if gammas is not None:
+            ref = ref * gammas[:, None]
+        ref = ref.to(torch.float16)
+    else:
+        ref = omoe.matmul(x, w, bias, sizes, gather_indx=gather, scatter_indx=scatter, gammas=gammas)
+    assert ref.dtype == torch.float16
+    assert_close(ref, y.cpu(), maxtol=2e-2, what="y")
+    assert_allclose_gate(ref, y.cpu(), what="y")
+
+
 @pytest.mark.parametrize("m, n, k, wkind", [(300, 512, 416, "bf16_kmajor"), (720, 576, 768, "mxfp4"), (40, 5760, 2880, "mxfp4"),
                                             (720, 576, 768, "mxfp4_tiled"), (900, 5760, 2880, "mxfp4_tiled")])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])

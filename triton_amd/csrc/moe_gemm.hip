@@ -48,7 +48,7 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 constexpr uint32_t kDroppedStore = 0x80000000u;
 typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
 
-enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3
+enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2, WK_F16 = 3 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3, fp16 (with fp16 activations)
 
 struct GemmParams {
   const uint8_t* x;    // bf16 or e4m3 rows
@@ -210,6 +210,25 @@ __device__ inline uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// output conversions of the shared epilogue: bf16, or fp16 for the fp16 x fp16 kernel
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_out2(float a, float b) {
+  if constexpr (F16) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  } else {
+    return pack_bf16x2(a, b);
+  }
+}
+template <bool F16>
+__device__ __forceinline__ uint16_t cvt_out(float a) {
+  if constexpr (F16)
+    return f32_to_f16_bits(a);
+  else
+    return f32_to_bf16_bits(a);
+}
+
 // FM = 16: v_mfma_f32_16x16x32_bf16 (lane = row % 16, 4 k-groups of 32 per 128-wide sub-stage).
 // FM = 32: v_mfma_f32_32x32x16_bf16 (lane = row % 32, 2 k-groups of 64), the full-rate shape on gfx950.
 template <int FM>
@@ -221,6 +240,10 @@ struct Frag<16> {
   static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
+  // the same registers read as eight fp16 values
+  static __device__ __forceinline__ acc_t mma_f16(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
   // accumulator register i of lane group h holds fragment row (= output column) n_of(i, h)
   static __device__ __forceinline__ int n_of(int i, int h) { return h * 4 + i; }
 };
@@ -231,6 +254,9 @@ struct Frag<32> {
   static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ acc_t mma_f16(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ int n_of(int i, int h) { return (i >> 2) * 8 + h * 4 + (i & 3); }
 };
 
@@ -238,7 +264,7 @@ struct Frag<32> {
 // ncol0 + f*FM) and row fragment j (tile rows (j*WM + mw)*FM ..); register i of a lane in lane group h holds
 // output column Frag::n_of(i, h) of row lr.  Order: row/column scales, bias, activation, gate weight,
 // (scattered) store.  Everything the rows and columns need from memory is fetched before the first store.
-template <int FM, int WM, int MFW, int NFW, bool SWIGLU>
+template <int FM, int WM, int MFW, int NFW, bool SWIGLU, bool F16OUT = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag<FM>::acc_t (&acc)[NFW][MFW], int expert,
                                               int off_m, int start_m, int eM, int ncol0, bool full_n, int mw, int lr, int h) {
   typedef Frag<FM> FR;
@@ -368,7 +394,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
           if (fast) {
             uint32_t w[VW / 4];
 #pragma unroll
-            for (int i = 0; i < VW / 4; ++i) w[i] = pack_bf16x2(r[2 * i], r[2 * i + 1]);
+            for (int i = 0; i < VW / 4; ++i) w[i] = pack_out2<F16OUT>(r[2 * i], r[2 * i + 1]);
             if constexpr (VW == 8)
               *reinterpret_cast<uint2*>(yrow + o0) = make_uint2(w[0], w[VW / 4 - 1]);
             else
@@ -376,13 +402,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
           } else {
 #pragma unroll
             for (int i = 0; i < VW / 2; ++i)
-              if (o0 + i < NOUT) yrow[o0 + i] = f32_to_bf16_bits(r[i]);
+              if (o0 + i < NOUT) yrow[o0 + i] = cvt_out<F16OUT>(r[i]);
           }
         } else {
           if (fast) {
             uint32_t w[VW / 2];
 #pragma unroll
-            for (int i = 0; i < VW / 2; ++i) w[i] = pack_bf16x2(v[f][u][2 * i] * g, v[f][u][2 * i + 1] * g);
+            for (int i = 0; i < VW / 2; ++i) w[i] = pack_out2<F16OUT>(v[f][u][2 * i] * g, v[f][u][2 * i + 1] * g);
             if constexpr (VW == 8)
               *reinterpret_cast<uint4*>(yrow + n0[f][u]) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
             else
@@ -390,7 +416,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
           } else {
 #pragma unroll
             for (int i = 0; i < VW; ++i)
-              if (n0[f][u] + i < N) yrow[n0[f][u] + i] = f32_to_bf16_bits(v[f][u][i] * g);
+              if (n0[f][u] + i < N) yrow[n0[f][u] + i] = cvt_out<F16OUT>(v[f][u][i] * g);
           }
         }
       }
@@ -659,7 +685,12 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
       for (int j = 0; j < MFW; ++j) {
         if (FULL || j < jcount) {
 #pragma unroll
-          for (int f = 0; f < NFW; ++f) acc[f][j] = FR::mma(wf[cur][f], xf[cur][j], acc[f][j]);
+          for (int f = 0; f < NFW; ++f) {
+            if constexpr (WK == WK_F16)
+              acc[f][j] = FR::mma_f16(wf[cur][f], xf[cur][j], acc[f][j]);
+            else
+              acc[f][j] = FR::mma(wf[cur][f], xf[cur][j], acc[f][j]);
+          }
         }
       }
       if constexpr (FULL) {
@@ -705,7 +736,7 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
     __syncthreads();
   }
 
-  gemm_epilogue<FM, WM, MFW, NFW, SWIGLU>(p, acc, expert, off_m, start_m, eM, n_tile + nw * NFW * FM, n_tile + BN <= N, mw, lr, h);
+  gemm_epilogue<FM, WM, MFW, NFW, SWIGLU, WK == WK_F16>(p, acc, expert, off_m, start_m, eM, n_tile + nw * NFW * FM, n_tile + BN <= N, mw, lr, h);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2466,11 +2497,14 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->M < 0 || d->N < 0 || d->K < 0) return fail(TK_ERR_INVALID, "tk_moe_gemm: negative size");
   if (d->M == 0 || d->N == 0 || d->grid_m == 0) return TK_OK;
   if (!d->x || !d->w || !d->y) return fail(TK_ERR_INVALID, "tk_moe_gemm: null operand");
-  if (d->x_dtype != TK_BF16 && d->x_dtype != TK_E4M3) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16 or e4m3 (dtype %d)", d->x_dtype);
+  const bool f16 = d->x_dtype == TK_F16 || d->w_dtype == TK_F16;  // fp16 x fp16 -> fp16, strided weights only
+  if (f16 && (d->x_dtype != TK_F16 || d->w_dtype != TK_F16 || d->y_dtype != TK_F16 || d->w_layout != TK_W_STRIDED || d->tile_counters || d->combine_counters))
+    return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: fp16 activations go with strided fp16 weights and an fp16 output");
+  if (d->x_dtype != TK_BF16 && d->x_dtype != TK_E4M3 && !f16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16, fp16 or e4m3 (dtype %d)", d->x_dtype);
   const bool mx_act = d->x_dtype == TK_E4M3 && d->x_mx_scale != nullptr;  // MXFP8 activations: scaled-MFMA path
   if (!mx_act && (d->x_dtype == TK_E4M3) != (d->w_dtype == TK_E4M3)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: e4m3 activations go with e4m3 weights, or with MX scales and tiled MXFP4 weights (x dtype %d, w dtype %d)", d->x_dtype, d->w_dtype);
   const bool mx_out = d->y_dtype == TK_E4M3 && d->y_mx_scale != nullptr;
-  if (d->y_dtype != TK_BF16 && !(mx_out && mx_act)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16, or e4m3 with y_mx_scale on the MXFP8-activation path (dtype %d)", d->y_dtype);
+  if (d->y_dtype != TK_BF16 && !f16 && !(mx_out && mx_act)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16, or e4m3 with y_mx_scale on the MXFP8-activation path (dtype %d)", d->y_dtype);
   if (d->activation != TK_ACT_NONE && d->activation != TK_ACT_SWIGLU) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad activation %d", d->activation);
   if (d->activation == TK_ACT_SWIGLU && d->N % 2) return fail(TK_ERR_INVALID, "tk_moe_gemm: swiglu needs an even N");
   const int xe = d->x_dtype == TK_E4M3 ? 16 : 8;  // elements per 16 bytes
@@ -2628,6 +2662,15 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     p.w_stride_e = d->w_stride_e * 2;
     p.w_stride_n = d->w_stride_n * 2;
     return launch_wk<WK_BF16>(p, d->block_m, d->grid_m, swiglu, st);
+  }
+  if (d->w_dtype == TK_F16) {
+    // fp16 x fp16 -> fp16 (v_mfma_f32_*_f16); same data path as bf16
+    if (d->x_dtype != TK_F16 || d->y_dtype != TK_F16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: fp16 weights go with fp16 activations and an fp16 output");
+    if (d->w_mx_scale) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: MX scales with fp16 weights");
+    if (d->w_stride_n % 8 || d->w_stride_e % 8 || (reinterpret_cast<uintptr_t>(d->w) & 15)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: weight columns must be 16-byte aligned");
+    p.w_stride_e = d->w_stride_e * 2;
+    p.w_stride_n = d->w_stride_n * 2;
+    return launch_wk<WK_F16>(p, d->block_m, d->grid_m, swiglu, st);
   }
   if (d->w_dtype == TK_E4M3) {
     if (d->w_mx_scale) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: MX scales with e4m3 weights");

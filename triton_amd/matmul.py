@@ -447,8 +447,11 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         has_limit = int(lim is not None)
         limit = float(lim) if lim is not None else 0.0
     out_dtype = precision_config.out_dtype or a.dtype
-    if out_dtype != torch.bfloat16 and not mx_out_fused:
-        raise NotImplementedError(f"output dtype {out_dtype} is not supported (bf16 only); set precision_config.out_dtype")
+    f16 = a.dtype == torch.float16 or w.dtype == torch.float16
+    if f16 and not (a.dtype == w.dtype == out_dtype == torch.float16 and not (tiled or tiled_fp8 or mx_act) and b_scale is None):
+        raise NotImplementedError(f"fp16 activations go with strided fp16 weights and an fp16 output (got {a.dtype} x {w.dtype} -> {out_dtype})")
+    if out_dtype != torch.bfloat16 and not mx_out_fused and not f16:
+        raise NotImplementedError(f"output dtype {out_dtype} is not supported (bf16, or fp16 for fp16 operands); set precision_config.out_dtype")
     y_rows = scatter_indx.shape[0] if scatter_indx is not None else M
     out_shape = (y_rows, N // reduction_n)
     c_scale = None
