@@ -159,6 +159,83 @@ def test_matmul_fp16(mods, device, m, n, k, mode, block_m, k_major, do_gather, d
     assert_allclose_gate(ref, y.cpu(), what="y")
 
 
+_NARROW = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2, "mxfp8_e4m3": torch.float8_e4m3fn,
+           "mxfp8_e5m2": torch.float8_e5m2, "mxfp4": torch.uint8}
+
+
+def _operand(t, kind, axis):
+    """(values, scales or None, what the operand means as a 16-bit tensor) for an operand kind of the reference's test
+    matrix (test_matmul.py:116-250)."""
+    if kind in ("bf16", "fp16"):
+        v = t.to(torch.bfloat16 if kind == "bf16" else torch.float16)
+        return v, None, v
+    if kind.startswith("mx"):
+        q, sc = omx.downcast_to_mxfp(t.to(torch.bfloat16), _NARROW[kind], axis=axis)
+        return q, sc, omx.upcast_from_mxfp(q, sc, torch.bfloat16, axis=axis)
+    q = t.to(_NARROW[kind])
+    return q, None, q.to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("m, n, k, mode, akind, wkind, tiled", [
+    (300, 400, 416, "ragged", "bf16", "mxfp8_e4m3", False),
+    (300, 400, 416, "ragged", "bf16", "mxfp8_e5m2", False),
+    (300, 400, 832, "ragged", "e5m2", "mxfp4", False),
+    (300, 400, 832, "ragged", "e5m2", "mxfp4", True),
+    (16, 256, 256, "ragged", "e5m2", "mxfp4", True),
+    (1024, 1024, 1024, "ragged", "e5m2", "mxfp4", True),
+    (300, 400, 416, "ragged", "e5m2", "mxfp8_e4m3", False),
+    (300, 400, 416, "ragged", "e5m2", "e5m2", False),
+    (600, 400, 416, "plain", "e5m2", "e5m2", False),
+    (300, 400, 416, "ragged", "e4m3", "mxfp4", False),
+    (300, 400, 416, "ragged", "mxfp8_e4m3", "mxfp8_e4m3", False),
+    (300, 400, 416, "ragged", "mxfp8_e5m2", "mxfp4", True),
+    (300, 400, 416, "ragged", "mxfp8_e4m3", "mxfp4", False),
+    (64, 128, 96, "ragged", "mxfp8_e4m3", "bf16", False),
+    (64, 128, 96, "ragged", "mxfp8_e4m3", "fp16", False),
+    (64, 128, 96, "ragged", "mxfp4", "bf16", False),
+    (64, 128, 96, "ragged", "mxfp4", "fp16", False),
+    (256, 256, 256, "plain", "mxfp4", "mxfp4", False),
+    (256, 256, 256, "plain", "mxfp4", "mxfp4", True),
+])
+@pytest.mark.parametrize("block_m", [16, 128])
+@pytest.mark.parametrize("do_gather, do_scatter, do_gamma", [(False, False, False), (True, True, True)])
+def test_expanded_operand_pairs(mods, device, m, n, k, mode, akind, wkind, tiled, block_m, do_gather, do_scatter, do_gamma):
+    """Operand pairs of the reference's matrix that run on the 16-bit kernels after the MX dequantiser has expanded the
+    narrow side; the oracle multiplies the same dequantised operands."""
+    mm, _, tensor = mods
+    g = torch.Generator().manual_seed(m + 3 * n + 7 * k + len(akind) * 11 + len(wkind))
+    n_slices = 10 if mode == "ragged" else 1
+    xv, xs, x_ref = _operand(torch.randn((m, k), generator=g), akind, -1)
+    wv, ws, w_ref = _operand(torch.randn((n_slices, k, n), generator=g) * 2 / k**0.5, wkind, 1)
+    if akind == "fp16" or wkind == "fp16":
+        x_ref, w_ref = x_ref.to(torch.float16), w_ref.to(torch.float16)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g) if mode == "ragged" else None
+    gather = torch.randint(0, m, (m, ), generator=g, dtype=torch.int32) if do_gather else None
+    scatter = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    gammas = 2.0**torch.randint(-5, 0, (m, ), generator=g).float() if do_gamma else None
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m) if sizes is not None else None
+    dev = lambda t: None if t is None else t.to(device)
+    wd, wsd = dev(wv), dev(ws)
+    if wkind == "mxfp4":
+        wd = tensor.wrap_torch_tensor(wd, dtype=tensor.FP4)
+        if tiled:
+            from triton_amd.tensor_details.layout import make_default_matmul_mxfp4_w_layout, make_default_matmul_mxfp4_w_scale_layout
+            wd = tensor.convert_layout(wd, make_default_matmul_mxfp4_w_layout(mx_axis=1))
+            wsd = tensor.convert_layout(tensor.wrap_torch_tensor(wsd), make_default_matmul_mxfp4_w_scale_layout(mx_axis=1))
+    xd = dev(xv)
+    if akind == "mxfp4":
+        xd = tensor.wrap_torch_tensor(xd, dtype=tensor.FP4)
+    pc = mm.PrecisionConfig(a_mx_scale=dev(xs), b_mx_scale=wsd)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(xd, wd, dev(bias) if mode == "ragged" else dev(bias[0]), md, gather_indx=dev(gather),
+                      scatter_indx=dev(scatter), precision_config=pc, gammas=dev(gammas))
+    assert y.dtype == x_ref.dtype
+    ref = omoe.matmul(x_ref, w_ref, bias, sizes, gather_indx=gather, scatter_indx=scatter, gammas=gammas)
+    assert_close(ref, y.cpu(), maxtol=3e-2 if wkind == "mxfp4" else 2e-2, what="y")
+    assert_allclose_gate(ref, y.cpu(), what="y")
+
+
 @pytest.mark.parametrize("m, n, k, wkind", [(300, 512, 416, "bf16_kmajor"), (720, 576, 768, "mxfp4"), (40, 5760, 2880, "mxfp4"),
                                             (720, 576, 768, "mxfp4_tiled"), (900, 5760, 2880, "mxfp4_tiled")])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])

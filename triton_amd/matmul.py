@@ -10,6 +10,11 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
                                                 ones are re-laid out once (the copy is cached on the tensor)
     bf16         mxfp4 (uint8 e2m1 + e8m0)      dequantised in registers, bf16 MFMA, fp32 accumulate
     fp8 e4m3     fp8 e4m3 (+ fp32 row/col scales via a/b_mx_tensor_scale)
+    mxfp8 e4m3   tiled mxfp4                    both operands in storage format on the scaled MFMA
+    fp16         fp16                           fp16 MFMA, fp16 output
+    other pairs of {bf16, fp16, e4m3, e5m2, mxfp8, mxfp4} activations x {bf16, fp16, e5m2, mxfp8, mxfp4} weights:
+                                                the narrow operand without a native partner is expanded to bf16 / fp16 by
+                                                the MX dequantiser kernel (activations per call, weights once, cached)
 
 Options of the reference signature that this build rejects with NotImplementedError: `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
 output / accumulator scales, split-k.  Batched 3-D activations run as a ragged problem with equal slices.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
@@ -18,6 +23,7 @@ MX quantiser kernel on the same stream.
 """
 from __future__ import annotations
 
+import dataclasses
 from dataclasses import dataclass
 from enum import Enum, auto
 from typing import Callable
@@ -137,6 +143,89 @@ def _combine_counters(device: torch.device) -> torch.Tensor:
 def _flex_out_is_trivial(flex: FlexCtx) -> bool:
     return (flex.acc_data.scale is None and flex.out_data.expected_scale is None and flex.out_data.actual_scale is None
             and flex.out_data.checksum_scale is None)
+
+
+_FP8_TYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
+
+
+def _strided_scale_data(scale) -> torch.Tensor:
+    """The e8m0 bytes of an MX scale operand in logical (strided) order."""
+    if isinstance(scale, Tensor):
+        if isinstance(scale.storage.layout, CDNA4MXScaleLayout):
+            scale = convert_layout(scale, StridedLayout(-2))
+        if not isinstance(scale.storage.layout, StridedLayout):
+            raise NotImplementedError(f"scale layout {type(scale.storage.layout).__name__} is not supported")
+        return scale.storage.data
+    return scale
+
+
+def _expanded_weights(w: torch.Tensor, scale, target: torch.dtype) -> torch.Tensor:
+    """fp8 weights (with or without e8m0 scales along K) as a 16-bit float tensor, converted by the MX dequantiser ONCE
+    and kept on the weight tensor (keyed by the version counters of values and scales)."""
+    from .numerics_details.mxfp import upcast_from_mxfp
+    sd = _strided_scale_data(scale) if scale is not None else None
+    key = (w._version, None if sd is None else (sd.data_ptr(), sd._version), target)
+    cached = getattr(w, "_tk_expanded", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    K = w.shape[-2]
+    if K % MXFP_BLOCK_SIZE:
+        raise NotImplementedError(f"fp8 weights that are expanded to {target} need K % 32 == 0 (got {K})")
+    if sd is None:
+        sd = torch.full((*w.shape[:-2], K // MXFP_BLOCK_SIZE, w.shape[-1]), 127, dtype=torch.uint8, device=w.device)
+    conv = upcast_from_mxfp(w, sd, target, axis=-2)
+    try:
+        w._tk_expanded = (key, conv)
+    except (AttributeError, RuntimeError):
+        pass
+    return conv
+
+
+def _expand_operands(a, b, precision_config):
+    """Operand pairs that have no kernel of their own run on the 16-bit kernels after the MX dequantiser kernel has
+    expanded the narrow operand (exact: an e2m1 / e4m3 / e5m2 value times a power of two is a bf16 value while it stays in
+    bf16's range, so the products the MFMA sees are those of the reference's in-kernel conversion):
+
+      * fp8 (e4m3 / e5m2) or MXFP8 / MXFP4 activations with weights other than the native partners (e4m3 x e4m3, and
+        MXFP8-e4m3 x tiled MXFP4 on the scaled MFMA) are expanded per call;
+      * MXFP8 weights (fp8 values + `b_mx_scale`) and plain e5m2 weights are expanded once and cached on the tensor.
+
+    Returns the (possibly replaced) operands and precision config."""
+    from .numerics_details.mxfp import upcast_from_mxfp
+    pc = precision_config
+    a_data = a.storage.data if isinstance(a, Tensor) else a
+    b_data = b.storage.data if isinstance(b, Tensor) else b
+    b_strided = not isinstance(b, Tensor) or isinstance(b.storage.layout, StridedLayout)
+    b_tiled_mx = isinstance(b, Tensor) and isinstance(b.storage.layout, GFX950MXValueLayout)
+    b_tiled_fp8 = isinstance(b, Tensor) and isinstance(b.storage.layout, GFX950FP8ValueLayout)
+    a_fp8 = a_data.dtype in _FP8_TYPES
+    a_mx = pc.a_mx_scale is not None
+    a_fp4 = a_mx and (a_data.dtype == torch.uint8 or (isinstance(a, Tensor) and a.dtype == FP4))
+    target = torch.float16 if torch.float16 in (a_data.dtype, b_data.dtype) else torch.bfloat16
+    if b_data.dtype in _FP8_TYPES and b_strided:
+        native = b_data.dtype == torch.float8_e4m3fn and pc.b_mx_scale is None and a_data.dtype == torch.float8_e4m3fn and not a_mx
+        if not native:
+            b = _expanded_weights(b_data, pc.b_mx_scale, target)
+            b_data = b
+            pc = dataclasses.replace(pc, b_mx_scale=None)
+    if a_fp8 or a_fp4:
+        native = (a_data.dtype == torch.float8_e4m3fn
+                  and ((a_mx and b_tiled_mx) or (not a_mx and (b_tiled_fp8 or b_data.dtype == torch.float8_e4m3fn))))
+        if not native:
+            if a_data.ndim != 2:
+                raise NotImplementedError("narrow activations that are expanded must be 2-D")
+            K = a_data.shape[-1] * (2 if a_fp4 else 1)
+            if K % MXFP_BLOCK_SIZE:
+                raise NotImplementedError(f"{a_data.dtype} activations with these weights need K % 32 == 0 (got {K})")
+            if a_mx:
+                sd = _strided_scale_data(pc.a_mx_scale)
+                assert sd.dtype == torch.uint8, f"Unsupported microscale dtype {sd.dtype}"
+            else:
+                sd = torch.full((a_data.shape[0], K // MXFP_BLOCK_SIZE), 127, dtype=torch.uint8, device=a_data.device)
+            a = upcast_from_mxfp(a_data, sd, target, axis=-1)
+            pc = dataclasses.replace(pc, a_mx_scale=None)
+    return a, b, pc
+
 
 
 def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
@@ -355,6 +444,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         fused_activation = FusedActivation(FnSpecs.default(), tuple())
     if epilogue is None:
         epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+    a, b, precision_config = _expand_operands(a, b, precision_config)
     # MXFP8 activations (`a_mx_scale`): e4m3 values with one e8m0 scale per 32 k, multiplied with tiled MXFP4 weights
     # on the scaled MFMA (triton_kernels/matmul.py:130-132,783-795)
     a_scale = precision_config.a_mx_scale
