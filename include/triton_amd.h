@@ -247,12 +247,13 @@ enum tk_activation {
 typedef struct tk_gemm_desc {
   /* activations: [rows, K], unit stride along K */
   const void* x;
-  int32_t x_dtype; /* TK_BF16, TK_E4M3 with x_row_scale (plain fp8), or TK_E4M3 with x_mx_scale (MXFP8) */
+  int32_t x_dtype; /* TK_BF16, TK_F16 (with TK_F16 weights and output), TK_E4M3 with x_row_scale (plain fp8), or TK_E4M3
+                    * with x_mx_scale (MXFP8) */
   int64_t x_stride_m;
   const float* x_row_scale; /* fp32 per row of x, read at the source row src(r), or NULL */
   /* weights: [E, K, N]; e2m1 is packed two per byte along K and the strides count bytes */
   const void* w;
-  int32_t w_dtype; /* TK_BF16, TK_E2M1 (needs w_mx_scale), TK_E4M3 */
+  int32_t w_dtype; /* TK_BF16, TK_F16 (strided layout only), TK_E2M1 (needs w_mx_scale), TK_E4M3 */
   int64_t w_stride_e, w_stride_k, w_stride_n;
   const void* w_mx_scale; /* uint8 e8m0 [E, K/32, N] or NULL */
   int64_t ws_stride_e, ws_stride_k, ws_stride_n;
@@ -279,7 +280,7 @@ typedef struct tk_gemm_desc {
   int32_t M, N, K; /* M: rows of the single slice when not ragged; N: columns of W; K: reduction */
   /* output [rows, N or N/2], unit stride along N */
   void* y;
-  int32_t y_dtype; /* TK_BF16, or TK_E4M3 with y_mx_scale */
+  int32_t y_dtype; /* TK_BF16, TK_F16 (fp16 operands), or TK_E4M3 with y_mx_scale */
   int64_t y_stride_m;
   int32_t activation; /* enum tk_activation */
   float act_alpha, act_limit;
