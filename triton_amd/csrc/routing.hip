@@ -9,7 +9,9 @@
 //                        word, ~expert in the low word, so ties go to the LOWER expert id).  The wave
 //                        also accumulates its private per-expert histogram in LDS and writes it out
 //                        as one row of `partials`.
-//   route_scan_kernel    ONE workgroup: per expert an exclusive prefix over the waves' histograms,
+//   route_scan_kernel    ONE workgroup: per expert an exclusive prefix over the workgroups' histogram totals
+//                        (route_topk_kernel sums its four waves' histograms; the scatter adds the earlier waves
+//                        of its own workgroup back),
 //                        the expert totals (`col_sum`), their exclusive scan (`col_offs`) and, if
 //                        asked, the whole ragged metadata (slice offsets, block offsets and block
 //                        schedules for block sizes 16..256).
@@ -144,6 +146,7 @@ struct TopkParams {
   uint32_t* bitmatrix;      // [words][T_pad] or null
   int64_t bm_stride_w;
   int32_t* partials;        // [units][E] or null
+  int32_t* wg_totals;       // [workgroups][E] (with partials): the histograms of a workgroup's waves summed
   int32_t rows_per_wave;
   int32_t* fill_a;          // [T*k] arrays preset to -1 (the two permutations and the gather index), or null
   int32_t* fill_b;
@@ -243,9 +246,19 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
     }
   }
   }
-  if (p.partials && row_begin < p.T) {
-    wave_sync();
-    for (int e = lane; e < E; e += 64) p.partials[(int64_t)unit * E + e] = hist_s[wave][e];
+  if (p.partials) {
+    if (row_begin < p.T) {
+      wave_sync();
+      for (int e = lane; e < E; e += 64) p.partials[(int64_t)unit * E + e] = hist_s[wave][e];
+    }
+    // the workgroup's total per expert: the scan walks these rows, a quarter as many as there are waves
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += kWaves * 64) {
+      int t = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) t += hist_s[w][e];
+      p.wg_totals[(int64_t)blockIdx.x * E + e] = t;
+    }
   }
 }
 
@@ -778,7 +791,8 @@ struct ScatterParams {
   int32_t n_rows_imm;
   const int32_t* n_rows_ptr;
   int32_t rows_per_wave;
-  const int32_t* partials;  // [units][E], exclusive over units
+  const int32_t* partials;  // [units][E]: every wave's own histogram
+  const int32_t* wg_prefix; // [workgroups][E]: entries of the expert in earlier workgroups (exclusive scan of the totals)
   const int32_t* col_offs;  // [E+1]
   int32_t* col_sorted;      // [T*k]
   int32_t* row_sorted;      // [T*k]
@@ -798,7 +812,17 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
   if (row_begin >= p.T) return;
   int row_end = row_begin + p.rows_per_wave;
   row_end = row_end < p.T ? row_end : p.T;
-  for (int e = lane; e < E; e += 64) base_s[wave][e] = p.col_offs[e] + p.partials[(int64_t)unit * E + e];
+  // first position of this wave's entries of expert e: the expert's offset, its entries in earlier workgroups and in
+  // the earlier waves of this one (all loads independent of each other)
+  for (int e = lane; e < E; e += 64) {
+    int b = p.col_offs[e] + p.wg_prefix[(int64_t)blockIdx.x * E + e];
+    int prev[kWaves - 1];
+#pragma unroll
+    for (int w = 0; w < kWaves - 1; ++w) prev[w] = w < wave ? p.partials[(int64_t)(blockIdx.x * kWaves + w) * E + e] : 0;
+#pragma unroll
+    for (int w = 0; w < kWaves - 1; ++w) b += prev[w];
+    base_s[wave][e] = b;
+  }
   wave_sync();
   const int64_t f_begin = (int64_t)row_begin * k, f_end = (int64_t)row_end * k;
   const int64_t n_valid = (int64_t)(n_rows < p.T ? n_rows : p.T) * k;
@@ -839,10 +863,10 @@ __global__ __launch_bounds__(kWaves * 64) void route_scatter_kernel(const Scatte
   }
 }
 
-// Rows one wave routes: one for small batches (latency), more as T grows so that the per-wave histograms the scan has
-// to walk stay at <= 1024 rows of the workspace (<= 512 when a row is long: E > 256).  A wave pays about 1.2 us per row
-// (a dependent chain of lane exchanges, alone on its SIMD), the scan one memory round trip per 16 workspace rows of a
-// run, so shorter waves and a longer workspace are the better trade up to here.
+// Rows one wave routes: one for small batches (latency), more as T grows so that the workspace stays small: at most
+// 1024 waves (512 when a row is long: E > 256), i.e. 256 / 128 rows of workgroup totals for the scan to walk.  A wave
+// pays about 1.2 us per row (a dependent chain of lane exchanges, alone on its SIMD); with 2048 waves the scan's longer
+// walk (512 rows: 16 us against 12) costs more than the shorter waves save.
 int rows_per_wave_for(int T, int E) {
   const int64_t max_units = E <= 256 ? 1024 : 512;
   int rpw = 1;
@@ -909,7 +933,7 @@ extern "C" int64_t tk_route_workspace_bytes(int32_t T, int32_t E) {
   const int rpw = rows_per_wave_for(T, E);
   const int64_t units = (T + rpw - 1) / rpw;
   const int64_t units_pad = (units + kWaves - 1) / kWaves * kWaves;
-  return (units_pad * E + (int64_t)E + 1) * 4;
+  return (units_pad * E + units_pad / kWaves * E + (int64_t)E + 1) * 4;  // wave histograms, workgroup totals, expert offsets
 }
 
 // One routing pass with the kernels' scratch memory at `workspace` (tk_route_workspace_bytes(T, E) bytes, every word
@@ -930,7 +954,8 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   const int units = (T + rpw - 1) / rpw;
   const int units_pad = (units + kWaves - 1) / kWaves * kWaves;
   int32_t* partials = static_cast<int32_t*>(workspace);
-  int32_t* col_offs = partials ? partials + (int64_t)units_pad * E : nullptr;
+  int32_t* wg_totals = partials ? partials + (int64_t)units_pad * E : nullptr;
+  int32_t* col_offs = partials ? wg_totals + (int64_t)(units_pad / kWaves) * E : nullptr;
 
   TopkParams tp;
   tp.logits = d->logits;
@@ -947,6 +972,7 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   tp.bitmatrix = static_cast<uint32_t*>(d->bitmatrix);
   tp.bm_stride_w = d->bitmatrix_stride_w;
   tp.partials = want_meta ? partials : nullptr;
+  tp.wg_totals = want_meta ? wg_totals : nullptr;
   tp.rows_per_wave = rpw;
   tp.fill_a = want_meta ? d->col_sorted_indx : nullptr;
   tp.fill_b = want_meta ? d->row_sorted_indx : nullptr;
@@ -995,7 +1021,7 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   ro.max_n_blocks = d->max_n_blocks;
   const int want_ragged = d->slice_offs != nullptr;
   if (want_ragged && (!d->block_offs || (!d->block_schedule && d->max_n_blocks > 0))) return fail(TK_ERR_INVALID, "tk_route: incomplete ragged outputs");
-  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, partials, units, E, d->col_sum, col_offs, want_ragged, ro);
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, wg_totals, units_pad / kWaves, E, d->col_sum, col_offs, want_ragged, ro);
   rc = check_launch("route_scan_kernel");
   if (rc != TK_OK) return rc;
 
@@ -1009,6 +1035,7 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   sp.n_rows_ptr = d->n_rows_ptr;
   sp.rows_per_wave = rpw;
   sp.partials = partials;
+  sp.wg_prefix = wg_totals;
   sp.col_offs = col_offs;
   sp.col_sorted = d->col_sorted_indx;
   sp.row_sorted = d->row_sorted_indx;
