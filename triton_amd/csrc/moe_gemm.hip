@@ -762,6 +762,8 @@ __global__ __launch_bounds__(WM * WN * 64) void moe_gemm_kernel(const GemmParams
 // NFW = column fragments per wave (tile width 128 * NFW): the activation tile is fetched from L2 once per column
 // tile, so wider tiles cut the L2 -> L1 traffic, which is what bounds this kernel at prefill shapes.
 // WD / XD = depth of the weight register ring (2 or 4) / of the activation staging registers (1 or 2).
+// Tail tiles: when at most four of a tile's column fragments lie below N (NFW = 2), wave w multiplies fragment w only
+// (its second fragment is loaded but neither converted nor multiplied, and its stores are dropped).
 // BLKM = rows of a row block in the ragged metadata (block_m).  A tile processes its block in passes of
 // BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 5 an expert of up to 160 rows is ONE tile (weights read
 // once, no nearly empty second tile) and only larger blocks take a second pass.
@@ -779,7 +781,9 @@ constexpr int kMetaSlices = 1024;
 // stores between two loads is the same on every path, so the compiler's vmcnt waits for loads issued BEFORE the
 // epilogue (the next unit's first operands) do not wait for these stores to drain.
 
-template <int G, int MFW, int NFW, bool SWIGLU>
+// NFV = leading column fragments of the wave that hold real columns; the others skip the arithmetic and issue their
+// stores with the dropped offset, so that the number of stores is the same on every path.
+template <int G, int MFW, int NFW, int NFV, bool SWIGLU>
 __device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc, const float* bias_s,
                                                 const float* gam_s, const int* dst_s, int ncol_tile, int ncol0, int grp, int lr, int h) {
   const int NOUT = SWIGLU ? p.N / 2 : p.N;
@@ -796,6 +800,13 @@ __device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&
     for (int f = 0; f < NFW; ++f)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
+        if (f >= NFV) {
+          if (SWIGLU)
+            __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{0u, 0u}, yrsrc, kDroppedStore, 0, 0);
+          else
+            __builtin_amdgcn_raw_buffer_store_b128(u32x4_t{0u, 0u, 0u, 0u}, yrsrc, kDroppedStore, 0, 0);
+          continue;
+        }
         // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i: after the two
         // lane halves exchange their 4-column groups a lane holds 8 consecutive columns from 16u + 8h
         float v[8];
@@ -879,6 +890,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   struct Unit {
     int expert, blk_off, blk_rows, pid_n, start_m, pass_off;
     bool valid;
+    bool tail;  // at most four column fragments of the tile lie below N: one per wave (NFW = 2)
   };
   auto tile_unit = [&](int pid) __attribute__((always_inline)) -> Unit {
     Unit u;
@@ -917,6 +929,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     u.blk_rows = __builtin_amdgcn_readfirstlane(u.blk_rows);
     u.pid_n = __builtin_amdgcn_readfirstlane(u.pid_n);
     u.start_m = __builtin_amdgcn_readfirstlane(u.start_m);
+    u.tail = NFW == 2 && nfr - u.pid_n * (BN / 32) <= 4;
     return u;
   };
   // the unit after `u`: its next pass, or the first pass of tile `pid_after` (-1: none)
@@ -974,7 +987,8 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     }
 #pragma unroll
     for (int f = 0; f < NFW; ++f) {
-      int F = u.pid_n * (BN / 32) + nw * NFW + f;
+      // (tail tiles: fragment nw of the tile is this wave's first, its second lies past N)
+      int F = u.pid_n * (BN / 32) + (u.tail ? nw + 4 * f : nw * NFW + f);
       F = F < nfr ? F : nfr - 1;  // fragments past N repeat the last one; their columns are dropped in the epilogue
       wbase[f] = p.w + (int64_t)u.expert * p.w_stride_e + (int64_t)F * nst * 2048;
       sbase[f] = p.w_scale + (int64_t)u.expert * p.ws_stride_e + (int64_t)F * nst * 128;
@@ -1072,8 +1086,9 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   // One K-stage.  NJ = row fragments with valid rows (compile-time so the MFMA list is straight-line code);
   // only the 2*NJ activation pieces per thread that cover those fragments are staged.  WS = weight ring slot
   // of this stage (= c % WD); the activation LDS buffer is WS & 1.
-  auto stage = [&](auto nj_c, auto gi_c, auto ws_c, int c) __attribute__((always_inline)) {
+  auto stage = [&](auto nj_c, auto gi_c, auto nf_c, auto ws_c, int c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
+    constexpr int NFV = decltype(nf_c)::value;  // column fragments of this wave that are multiplied (the loads always cover NFW)
     constexpr int WS4 = decltype(ws_c)::value;  // c % 4
     constexpr int PAR = WS4 & 1;
     using WSC = template_int<WS4 % WD>;                // this stage's weights
@@ -1082,27 +1097,27 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     constexpr int XS = (WS4 + 1) % XD;                 // activation register slot holding X(c+1)
     constexpr int WLOAD_STEP = WD == 2 ? 0 : 4;        // the refilled slot was last read in step 6 of stage c-1
     constexpr int GI = decltype(gi_c)::value;  // this wave's row group
-    constexpr int NM = NJ * NFW;
+    constexpr int NM = NJ * NFV;
     // pieces to stage: a piece covers 16 rows (G = 1) or 32 rows (G = 2); with G = 2 the tile has 2*NJ - 1 or 2*NJ
     // (group 0), 2*NJ or 2*NJ + 1 (group 1) fragments with valid rows, and the larger count is staged
     constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
     constexpr int PPS = (NP + 3) / 4;    // per step, during steps 0..3
-    constexpr int NOPS = NJ + NFW + 4;   // NJ LDS reads, NFW conversions, three staging slots, the weight loads
+    constexpr int NOPS = NJ + NFV + 4;   // NJ LDS reads, NFV conversions, three staging slots, the weight loads
     static_for<0, 8>([&](auto t_c) __attribute__((always_inline)) {
       constexpr int t = decltype(t_c)::value;
       constexpr int cur = t & 1, nxt = cur ^ 1;
       auto op = [&](auto o_c) __attribute__((always_inline)) {
         constexpr int o = decltype(o_c)::value;
-        if constexpr (o == NJ + NFW + 3) {
+        if constexpr (o == NJ + NFV + 3) {
           if constexpr (t == WLOAD_STEP) load_w(WSL{}, c + WD - 1);
         } else if constexpr (t < 7) {
           if constexpr (o < NJ) {
             read_xf(PAR, t + 1, o, xf[nxt]);
-          } else if constexpr (o < NJ + NFW) {
+          } else if constexpr (o < NJ + NFV) {
             make_wf(WSC{}, t + 1, o - NJ, wf[nxt]);
           } else if constexpr (t < 4) {
             // next stage's activations: registers -> LDS, then refill the registers for a later stage
-            constexpr int half = o - NJ - NFW;
+            constexpr int half = o - NJ - NFV;
             constexpr int j = t * PPS + half;
             if constexpr (half < PPS && j < NP) {
               store_x_piece(j, PAR ^ 1, XS);
@@ -1112,7 +1127,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
         } else {
           if constexpr (o < NJ) {
             read_xf(PAR ^ 1, 0, o, xf[nxt]);
-          } else if constexpr (o < NJ + NFW) {
+          } else if constexpr (o < NJ + NFV) {
             make_wf(WSN{}, 0, o - NJ, wf[nxt]);
           }
         }
@@ -1129,7 +1144,7 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
       }
       static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
         constexpr int m = decltype(m_c)::value;
-        constexpr int j = m / NFW, f = m % NFW;
+        constexpr int j = m / NFV, f = m % NFV;
         acc[f][j] = FR::mma(wf[cur][f], xf[cur][j], acc[f][j]);
         if constexpr (t == 7 && m == 0) {
           // every wave has fetched its last operands of this buffer (during step 6) and written its share
@@ -1156,9 +1171,10 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
   int up = 0;             // operand set of the current unit
   Unit cur_unit;          // the unit being computed
   int resolve_slot = -1;  // thread 0 writes the claimed tile id into next_tile_s[resolve_slot] before the first barrier
-  auto run = [&](auto nj_c, auto gi_c) __attribute__((always_inline)) {
+  auto run = [&](auto nj_c, auto gi_c, auto nf_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
     constexpr int GI = decltype(gi_c)::value;
+    constexpr int NFV = decltype(nf_c)::value;
     constexpr int NP = G == 1 ? 2 * NJ : (2 * NJ + GI < XCH ? 2 * NJ + GI : XCH);
     // Prologue: finish stage 0 (its loads were issued by first_loads before the previous unit's epilogue).  The order
     // of the loads left in flight (activations, then weights, of stage 1, then of stage 2) is pinned to the order the
@@ -1189,32 +1205,42 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { read_xf(0, 0, decltype(jc)::value, xf[0]); });
-    static_for<0, NFW>([&](auto fc) __attribute__((always_inline)) { make_wf(S0, 0, decltype(fc)::value, wf[0]); });
+    static_for<0, NFV>([&](auto fc) __attribute__((always_inline)) { make_wf(S0, 0, decltype(fc)::value, wf[0]); });
     __builtin_amdgcn_sched_barrier(0);
     // all stages of a group always run inside the loop: a path that skips some and returns to the loop header
     // would again make the header's wait counts cover the loads just issued
     int c = 0;
     for (; c + 3 < nst; c += 4) {
-      stage(nj_c, gi_c, S0, c);
-      stage(nj_c, gi_c, S1, c + 1);
-      stage(nj_c, gi_c, S2, c + 2);
-      stage(nj_c, gi_c, S3, c + 3);
+      stage(nj_c, gi_c, nf_c, S0, c);
+      stage(nj_c, gi_c, nf_c, S1, c + 1);
+      stage(nj_c, gi_c, nf_c, S2, c + 2);
+      stage(nj_c, gi_c, nf_c, S3, c + 3);
     }
-    if (c < nst) stage(nj_c, gi_c, S0, c);
-    if (c + 1 < nst) stage(nj_c, gi_c, S1, c + 1);
-    if (c + 2 < nst) stage(nj_c, gi_c, S2, c + 2);
+    if (c < nst) stage(nj_c, gi_c, nf_c, S0, c);
+    if (c + 1 < nst) stage(nj_c, gi_c, nf_c, S1, c + 1);
+    if (c + 2 < nst) stage(nj_c, gi_c, nf_c, S2, c + 2);
   };
-  auto dispatch = [&](auto gi_c, int nj) __attribute__((always_inline)) {
+  auto dispatch = [&](auto gi_c, auto nf_c, int nj) __attribute__((always_inline)) {
     constexpr int GI = decltype(gi_c)::value;
     if constexpr (GI == 1) {
       if (nj == 0) {
-        run(template_int<0>{}, gi_c);
+        run(template_int<0>{}, gi_c, nf_c);
         return;
       }
     }
     static_for<1, MFW + 1>([&](auto n_c) __attribute__((always_inline)) {
-      if (nj == decltype(n_c)::value) run(n_c, gi_c);
+      if (nj == decltype(n_c)::value) run(n_c, gi_c, nf_c);
     });
+  };
+  // (tail tiles multiply one fragment per wave)
+  auto dispatch_nf = [&](auto gi_c, bool tail, int nj) __attribute__((always_inline)) {
+    if constexpr (NFW == 2) {
+      if (tail) {
+        dispatch(gi_c, template_int<1>{}, nj);
+        return;
+      }
+    }
+    dispatch(gi_c, template_int<NFW>{}, nj);
   };
 
   if (pid >= 0) {
@@ -1244,16 +1270,18 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
       const int nj = (nfrag_m - grp + G - 1) / G;  // those of this wave: tile fragments grp, grp + G, ...
       if constexpr (G == 2) {
         if (grp == 1)
-          dispatch(template_int<1>{}, nj);
+          dispatch_nf(template_int<1>{}, cur.tail, nj);
         else
-          dispatch(template_int<0>{}, nj);
+          dispatch_nf(template_int<0>{}, cur.tail, nj);
       } else {
-        dispatch(template_int<0>{}, nj);
+        dispatch_nf(template_int<0>{}, cur.tail, nj);
       }
       resolve_slot = -1;
 
       // ---- before this unit's epilogue: everything the next units need from memory ----
-      const int ncol0 = cur.pid_n * BN + nw * NFW * FM;
+      const int wcol = cur.tail ? nw * FM : nw * NFW * FM;  // this wave's first column in the tile
+      const int ncol0 = cur.pid_n * BN + wcol;
+      const bool cur_tail = cur.tail;
       Unit nxt2 = nxt;
       if (nxt.valid) {
         if (cur.pass_off + BM >= cur.blk_rows) {
@@ -1282,7 +1310,10 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
         unit_pointers(nxt, up);
         first_loads();
       }
-      staged_epilogue<G, MFW, NFW, SWIGLU>(p, acc, yrsrc, bias_s[up], gam_s[up], dst_s[up], nw * NFW * FM, ncol0, grp, lr, h);
+      if (NFW == 2 && cur_tail)
+        staged_epilogue<G, MFW, NFW, 1, SWIGLU>(p, acc, yrsrc, bias_s[up], gam_s[up], dst_s[up], wcol, ncol0, grp, lr, h);
+      else
+        staged_epilogue<G, MFW, NFW, NFW, SWIGLU>(p, acc, yrsrc, bias_s[up], gam_s[up], dst_s[up], wcol, ncol0, grp, lr, h);
       if (!nxt.valid) break;
       cur = nxt;
       nxt = nxt2;
