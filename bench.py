@@ -114,6 +114,43 @@ def spin_up(fn, seconds=0.15):
         torch.cuda.synchronize()
 
 
+def board_state_under(fn, seconds=2.5):
+    """Socket power and engine clocks as `amd-smi` reports them while `fn` keeps the GPU busy (launched in a loop from
+    this thread while a second thread asks amd-smi once, a second into the load).  The published peaks assume 2.4 GHz;
+    what the board sustains under a kernel at its power cap is part of reading a roofline fraction.  None when amd-smi
+    is missing, fails, or a profiler is attached (its preloaded library would follow into the child process)."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    if shutil.which("amd-smi") is None or "rocprof" in os.environ.get("LD_PRELOAD", ""):
+        return None
+    out = {}
+
+    def ask():
+        time.sleep(1.0)
+        try:
+            r = subprocess.run(["amd-smi", "metric", "--clock", "--power", "--json"], capture_output=True, text=True, timeout=20)
+            pw = re.search(r'"socket_power":\s*\{\s*"value":\s*(\d+)', r.stdout)
+            clks = re.findall(r'"gfx_\d+":\s*\{\s*"clk":\s*\{\s*"value":\s*(\d+)', r.stdout)
+            if pw and clks:
+                out["socket_power_w"] = int(pw.group(1))
+                out["gfx_mhz_min"] = min(int(c) for c in clks)
+                out["gfx_mhz_max"] = max(int(c) for c in clks)
+        except Exception:  # noqa: BLE001  (a figure for the report, never a reason to fail the bench)
+            pass
+
+    th = threading.Thread(target=ask)
+    th.start()
+    t0 = time.perf_counter()
+    while th.is_alive() and time.perf_counter() - t0 < 30.0:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+    th.join()
+    return out or None
+
+
 def time_steps(fn, steps, warmup):
     spin_up(fn)
     for _ in range(warmup):
@@ -298,9 +335,10 @@ def bench_fp8(device, steps, warmup):
         return reduce(y.view(T, k, -1), dim=1)[0]
 
     ms = time_steps(step, steps, warmup)
+    board = board_state_under(step)
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
     return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8",
-                frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4))
+                frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), board_under_step=board)
 
 
 def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
@@ -331,6 +369,7 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
         return reduce(y.view(T, k, -1), dim=1)[0]
 
     ms = time_steps(step, steps, warmup)
+    board = board_state_under(step)
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
     # algorithmic bytes with one-byte activations: x_q + scales, W1, h_q twice, W2, y twice, out
     R = T * k
@@ -339,7 +378,7 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
     t_roof_ms = max(flops / 5.0e15, nbytes / (PEAK_HBM_GBPS * 1e9)) * 1e3
     return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8 (MXFP8 x MXFP4, scaled MFMA)",
                 frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), t_roof_ms=round(t_roof_ms, 4), frac=round(t_roof_ms / ms, 4),
-                bound="hbm" if nbytes / (PEAK_HBM_GBPS * 1e9) > flops / 5.0e15 else "mfma")
+                bound="hbm" if nbytes / (PEAK_HBM_GBPS * 1e9) > flops / 5.0e15 else "mfma", board_under_step=board)
 
 
 def main():
@@ -349,6 +388,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the decode and MX round-trip figures")
+    ap.add_argument("--no-board-state", action="store_true", help="do not sample amd-smi (power, clocks) under the dominant kernel")
     ap.add_argument("--calibrate-copy", action="store_true", help="also run a 1 GiB device copy (reference kernel for counter runs)")
     ap.add_argument("--only", choices=["mx", "decode", "fp8", "ragged_k"],
                     help="run one of the side workloads alone and print its figures (for profiler runs)")
@@ -416,6 +456,7 @@ def main():
     e1.record()
     torch.cuda.synchronize()
     gemm1_ms = e0.elapsed_time(e1) / args.steps
+    board = None if args.no_board_state else board_state_under(gemm1)
     ms_eager = time_steps(lambda: layer(x, logits), args.steps, args.warmup)
     R = T * k
     flops1 = 2.0 * R * d * f2
@@ -440,7 +481,8 @@ def main():
                    "experts": E, "top_k": k, "w1": [E, d, f2], "w2": [E, f2 // 2, d]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM1_TRAFFIC_BYTES,
-                     "kernel": "moe_gemm_mxn_kernel (gather-GEMM, tiled MXFP4 W1, bias, swiglu)", "kernel_ms": round(gemm1_ms, 4)},
+                     "kernel": "moe_gemm_mxn_kernel (gather-GEMM, tiled MXFP4 W1, bias, swiglu)", "kernel_ms": round(gemm1_ms, 4),
+                     "board_under_kernel": board},
     }
     # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
     layer_bytes = 2.19e9
