@@ -151,6 +151,32 @@ def board_state_under(fn, seconds=2.5):
     return out or None
 
 
+def mfma_sustained_probe(device):
+    """bf16 MFMA rate the board sustains under its power cap: a kernel of nothing but v_mfma_f32_32x32x16_bf16 on
+    register operands (tk_probe_mfma_bf16), timed with events, with amd-smi's power and clocks under it.  The published
+    2.5 PFLOP/s assumes 2.4 GHz; this is the ceiling a bf16 GEMM can be held against on this machine."""
+    from triton_amd import _native as nt
+    n_wg = 2 * torch.cuda.get_device_properties(device).multi_processor_count
+    iters = 4000
+    out = torch.zeros(n_wg * 256, dtype=torch.float32, device=device)
+
+    def fn():
+        with nt.on_device(device):
+            nt.check(nt.lib().tk_probe_mfma_bf16(out.data_ptr(), n_wg, iters, nt.stream_ptr(device)))
+
+    spin_up(fn, 0.5)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / 20
+    flops = n_wg * 4 * iters * 8 * 32768.0
+    return dict(TFLOPs=round(flops / ms / 1e9, 1), frac_of_published_peak=round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                board=board_state_under(fn))
+
+
 def time_steps(fn, steps, warmup):
     spin_up(fn)
     for _ in range(warmup):
@@ -482,7 +508,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM1_TRAFFIC_BYTES,
                      "kernel": "moe_gemm_mxn_kernel (gather-GEMM, tiled MXFP4 W1, bias, swiglu)", "kernel_ms": round(gemm1_ms, 4),
-                     "board_under_kernel": board},
+                     "board_under_kernel": board,
+                     "mfma_sustained_probe": None if args.no_board_state else mfma_sustained_probe(device)},
     }
     # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
     layer_bytes = 2.19e9

@@ -394,6 +394,14 @@ int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t
                                void* dx, tk_stream_t stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): a kernel of nothing but v_mfma_f32_32x32x16_bf16 on register
+ * operands, `n_workgroups` workgroups of four waves, `iters` x 8 instructions per wave (8 * 32768 FLOP * iters per wave).
+ * bench.py times it to report the bf16 MFMA rate this board sustains under its power cap.  `out`: at least
+ * n_workgroups * 256 floats of device memory (practically never written).
+ */
+int32_t tk_probe_mfma_bf16(float* out, int32_t n_workgroups, int32_t iters, tk_stream_t stream);
+
+/*
  * Per-row dynamic quantisation of bf16 activations to OCP e4m3: scales[m] = amax_m / 448 (1 for a zero
  * row), q[m, :] = saturating_cast(x[m, :] / scales[m]).  No counterpart kernel in the reference: its
  * benchmark casts activations to fp8 with a plain torch `.to()` (python/triton_kernels/bench/bench_mlp.py:169);

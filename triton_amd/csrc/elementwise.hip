@@ -154,10 +154,47 @@ int grid_for(int64_t total) {
   return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
 }
 
+// Measurement aid: nothing but v_mfma_f32_32x32x16_bf16 on register operands, eight independent accumulators per wave,
+// one wave per SIMD.  Its rate under the board's power cap is the ceiling a bf16 GEMM can be compared with on this
+// machine (the published peak assumes the 2.4 GHz engine clock, which the cap does not sustain under MFMA load).
+// Operands are lane-dependent, finite and of mixed sign so that the multipliers toggle as they do on real data.
+__global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(float* out, int iters) {
+  bf16x8_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int t = (int)threadIdx.x * 8 + e + 37 * i;
+      a[i][e] = (__bf16)(((t * 2654435761u >> 20) & 0xFF) * (1.0f / 128.0f) - 1.0f);
+      b[i][e] = (__bf16)(((t * 40503u >> 7) & 0xFF) * (1.0f / 128.0f) - 1.0f);
+    }
+  f32x16_t acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j & 3], b[(j >> 1) & 3], acc[j], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sum += acc[j][e];
+  if (sum == 123456.789f) out[blockIdx.x * 256 + threadIdx.x] = sum;  // keeps the loop; practically never true
+}
+
 }  // namespace
 }  // namespace tk
 
 using namespace tk;
+
+extern "C" int32_t tk_probe_mfma_bf16(float* out, int32_t n_workgroups, int32_t iters, tk_stream_t stream) {
+  if (!out || n_workgroups <= 0 || iters <= 0) return fail(TK_ERR_INVALID, "tk_probe_mfma_bf16: bad arguments");
+  hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3((unsigned)n_workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), out, iters);
+  return check_launch("probe_mfma_bf16_kernel");
+}
 
 extern "C" int32_t tk_swiglu(const void* a, int32_t dtype, int64_t M, int64_t n_out, int64_t stride_am, void* out,
                              int64_t stride_om, float alpha, float limit, int32_t has_limit, const int32_t* n_rows_ptr,
