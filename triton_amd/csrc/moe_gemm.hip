@@ -87,7 +87,7 @@ struct GemmParams {
   int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
   int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
   int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
-  int32_t* tile_counters;  // persistent kernels: kTileCounterWords zeroed words for dynamic tile claiming, or null
+  int32_t* tile_counters;  // persistent kernels: 16 zeroed words for dynamic tile claiming (9 are used), or null
   uint32_t y_bytes;        // persistent MXFP4 kernels: bytes of the output buffer that rows may be written to (< 2 GiB)
   int32_t combine_k;          // decode kernel: > 0 = sum the k rows of every token into combine_out (fused top-k combine)
   uint16_t* combine_out;      // bf16 [tokens, N]
@@ -108,7 +108,6 @@ struct GemmParams {
 // read when it ends, so the atomic's latency is hidden behind the tile's K loop.  Words 0..7 = next index of each
 // queue, word 8 = workgroups that have finished; the last one to finish clears all nine words, so the counters
 // are zero again when the kernel ends (launches that share the words must not overlap in time).
-constexpr int kTileCounterWords = 16;
 
 struct TileClaimer {
   int32_t* ctr;
@@ -139,8 +138,11 @@ struct TileClaimer {
   // would make every lane wait for the atomic to return right here)
   __device__ __forceinline__ void issue() {
     int fresh;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wsometimes-uninitialized"
     if (threadIdx.x == 0) fresh = atomicAdd(&ctr[myq], 1);
     pending = fresh;
+#pragma clang diagnostic pop
   }
   // thread 0: tile id of the claim in flight, or of another queue when the own one is exhausted; -1 = no tile left.
   // The other queues' counters are read together first, so a workgroup that finds everything taken pays two

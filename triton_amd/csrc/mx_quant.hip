@@ -462,7 +462,7 @@ __global__ __launch_bounds__(kThreads) void mx_down_tile(const uint16_t* __restr
                                                          int64_t L, int64_t inner, int64_t inner_last, int64_t col_tiles,
                                                          int64_t blk_tiles, uint8_t* __restrict__ out_vals,
                                                          uint8_t* __restrict__ out_scales, int rounding) {
-  constexpr int BB = TileGeom<KIND>::BB, NB = TileGeom<KIND>::NB;
+  constexpr int NB = TileGeom<KIND>::NB;
   __shared__ __attribute__((aligned(16))) uint8_t vals_s[kTileRows * kTilePitch];
   __shared__ uint8_t sc_s[kTileCols * NB];
   int64_t bid = tile_order(blockIdx.x, gridDim.x);
