@@ -281,6 +281,8 @@ def bench_decode(device, steps, warmup):
         gbytes = active * per_expert / 1e9
         res[f"T{T}"] = dict(ms=round(ms, 4), ms_eager=round(ms_eager, 4), active_experts=active, weight_GB=round(gbytes, 4),
                             GBps=round(gbytes / (ms * 1e-3), 1), frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
+        if T == 16:
+            res[f"T{T}"]["board_under_replay"] = board_state_under(graph.replay)
         del graph
     return res
 
@@ -293,9 +295,10 @@ def bench_mx(device, steps, warmup):
     ms_q = time_steps(lambda: downcast_to_mxfp(w, torch.uint8, axis=1), steps, warmup)
     q, s = downcast_to_mxfp(w, torch.uint8, axis=1)
     ms_d = time_steps(lambda: upcast_from_mxfp(q, s, torch.bfloat16, axis=1), steps, warmup)
+    board = board_state_under(lambda: downcast_to_mxfp(w, torch.uint8, axis=1))
     return dict(quant_ms=round(ms_q, 4), quant_GBps=round(nbytes / ms_q / 1e6, 1), dequant_ms=round(ms_d, 4),
                 dequant_GBps=round(nbytes / ms_d / 1e6, 1), frac_hbm_quant=round(nbytes / ms_q / 1e6 / PEAK_HBM_GBPS, 4),
-                frac_hbm_dequant=round(nbytes / ms_d / 1e6 / PEAK_HBM_GBPS, 4))
+                frac_hbm_dequant=round(nbytes / ms_d / 1e6 / PEAK_HBM_GBPS, 4), board_under_quant=board)
 
 
 def bench_ragged_k(device, steps, warmup):
