@@ -394,12 +394,13 @@ int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t
                                void* dx, tk_stream_t stream);
 
 /*
- * Measurement aid (no counterpart in the reference): a kernel of nothing but v_mfma_f32_32x32x16_bf16 on register
- * operands, `n_workgroups` workgroups of four waves, `iters` x 8 instructions per wave (8 * 32768 FLOP * iters per wave).
- * bench.py times it to report the bf16 MFMA rate this board sustains under its power cap.  `out`: at least
- * n_workgroups * 256 floats of device memory (practically never written).
+ * Measurement aid (no counterpart in the reference): a kernel of nothing but MFMA instructions on register operands,
+ * `n_workgroups` workgroups of four waves, `iters` x 8 instructions per wave: v_mfma_f32_32x32x16_bf16 (32768 FLOP each)
+ * or, with `fp8` != 0, v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP each).  bench.py times it to report the
+ * MFMA rates this board sustains under its power cap.  `out`: at least n_workgroups * 256 floats of device memory
+ * (practically never written).
  */
-int32_t tk_probe_mfma_bf16(float* out, int32_t n_workgroups, int32_t iters, tk_stream_t stream);
+int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t fp8, tk_stream_t stream);
 
 /*
  * Per-row dynamic quantisation of bf16 activations to OCP e4m3: scales[m] = amax_m / 448 (1 for a zero

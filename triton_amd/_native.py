@@ -93,7 +93,7 @@ SIGNATURES = {
     "tk_ragged_remap": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32, _i32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
     "tk_moe_gemm": (_i32, [_c.POINTER(GemmDesc), _ptr]),
     "tk_ragged_k_gemm": (_i32, [_c.POINTER(RaggedKDesc), _ptr]),
-    "tk_probe_mfma_bf16": (_i32, [_ptr, _i32, _i32, _ptr]),
+    "tk_probe_mfma": (_i32, [_ptr, _i32, _i32, _i32, _ptr]),
     "tk_swiglu": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _f32, _f32, _i32, _ptr, _ptr]),
     "tk_reduce_mid": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "tk_reduce_mid_backward": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),

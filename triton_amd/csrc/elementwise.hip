@@ -154,19 +154,23 @@ int grid_for(int64_t total) {
   return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
 }
 
-// Measurement aid: nothing but v_mfma_f32_32x32x16_bf16 on register operands, eight independent accumulators per wave,
-// one wave per SIMD.  Its rate under the board's power cap is the ceiling a bf16 GEMM can be compared with on this
-// machine (the published peak assumes the 2.4 GHz engine clock, which the cap does not sustain under MFMA load).
-// Operands are lane-dependent, finite and of mixed sign so that the multipliers toggle as they do on real data.
-__global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(float* out, int iters) {
-  bf16x8_t a[4], b[4];
+// Measurement aid: nothing but MFMA instructions on register operands, eight independent accumulators per wave, one
+// or two waves per SIMD.  Its rate under the board's power cap is the ceiling a GEMM of that MFMA class can be compared
+// with on this machine (the published peaks assume the 2.4 GHz engine clock, which the cap does not sustain under MFMA
+// load).  Operands are lane-dependent, finite and of mixed sign so that the multipliers toggle as they do on real data.
+// FP8 = false: v_mfma_f32_32x32x16_bf16 (32768 FLOP); true: v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP).
+typedef int i32x8_probe_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_probe __attribute__((ext_vector_type(4)));
+template <bool FP8>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters) {
+  uint32_t raw[4][8];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int t = (int)threadIdx.x * 8 + e + 37 * i;
-      a[i][e] = (__bf16)(((t * 2654435761u >> 20) & 0xFF) * (1.0f / 128.0f) - 1.0f);
-      b[i][e] = (__bf16)(((t * 40503u >> 7) & 0xFF) * (1.0f / 128.0f) - 1.0f);
+      const uint32_t t = ((uint32_t)threadIdx.x * 8u + e + 37u * i) * 2654435761u;
+      // bf16 pairs / e4m3 quads with exponents near 1.0 (no NaN or infinity patterns)
+      raw[i][e] = FP8 ? ((t & 0x87878787u) | 0x30303030u) : ((t & 0x807F807Fu) | 0x3F003F00u);
     }
   f32x16_t acc[8];
 #pragma unroll
@@ -175,7 +179,20 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(float* out, int it
     for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j & 3], b[(j >> 1) & 3], acc[j], 0, 0, 0);
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (FP8) {
+        const i32x8_probe_t a = {(int)raw[j & 3][0], (int)raw[j & 3][1], (int)raw[j & 3][2], (int)raw[j & 3][3],
+                                 (int)raw[j & 3][4], (int)raw[j & 3][5], (int)raw[j & 3][6], (int)raw[j & 3][7]};
+        const int bi = (j >> 1) & 3;
+        const i32x8_probe_t b = {(int)raw[bi][7], (int)raw[bi][6], (int)raw[bi][5], (int)raw[bi][4],
+                                 (int)raw[bi][3], (int)raw[bi][2], (int)raw[bi][1], (int)raw[bi][0]};
+        acc[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[j], 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      } else {
+        const u32x4_probe a = {raw[j & 3][0], raw[j & 3][1], raw[j & 3][2], raw[j & 3][3]};
+        const u32x4_probe b = {raw[(j >> 1) & 3][4], raw[(j >> 1) & 3][5], raw[(j >> 1) & 3][6], raw[(j >> 1) & 3][7]};
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc[j], 0, 0, 0);
+      }
+    }
   }
   float sum = 0.f;
 #pragma unroll
@@ -190,10 +207,14 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(float* out, int it
 
 using namespace tk;
 
-extern "C" int32_t tk_probe_mfma_bf16(float* out, int32_t n_workgroups, int32_t iters, tk_stream_t stream) {
-  if (!out || n_workgroups <= 0 || iters <= 0) return fail(TK_ERR_INVALID, "tk_probe_mfma_bf16: bad arguments");
-  hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3((unsigned)n_workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), out, iters);
-  return check_launch("probe_mfma_bf16_kernel");
+extern "C" int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t fp8, tk_stream_t stream) {
+  if (!out || n_workgroups <= 0 || iters <= 0) return fail(TK_ERR_INVALID, "tk_probe_mfma: bad arguments");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (fp8)
+    hipLaunchKernelGGL(probe_mfma_kernel<true>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
+  else
+    hipLaunchKernelGGL(probe_mfma_kernel<false>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
+  return check_launch("probe_mfma_kernel");
 }
 
 extern "C" int32_t tk_swiglu(const void* a, int32_t dtype, int64_t M, int64_t n_out, int64_t stride_am, void* out,
