@@ -1703,8 +1703,10 @@ __global__ __launch_bounds__(256) void moe_gemm_f8n_kernel(const GemmParams p) {
   __shared__ int next_tile_s[2];  // written by thread 0 before a tile's first barrier: the id of the tile after it
   int tile_par = 0, n_tile = 0;
   // (claiming needs at least one workgroup per XCD queue: a queue's tiles are reached through the workgroups that
-  // start on it)
-  const bool dyn = p.tile_counters != nullptr && gridDim.x >= 8;
+  // start on it.  With many rounds, or tiles that divide evenly among the workgroups, the static rounds are kept: a
+  // partly filled last round then costs little, while tiles that start together walk K in step and find each other's
+  // operands in the XCD's L2 — 4 % faster at 8192 tokens x top-2 of 8 experts, 56 rounds.)
+  const bool dyn = p.tile_counters != nullptr && gridDim.x >= 8 && live % (int)gridDim.x != 0 && live < 32 * (int)gridDim.x;
   TileClaimer claimer;
   int pid = claimer.init(p.tile_counters, live), round0 = 0;
   // (dynamic: a workgroup whose queue is shorter than its first index gets no tile at all, which only happens when
