@@ -151,19 +151,20 @@ def board_state_under(fn, seconds=2.5):
     return out or None
 
 
-def mfma_sustained_probe(device, fp8=False):
-    """MFMA rate the board sustains under its power cap: a kernel of nothing but v_mfma_f32_32x32x16_bf16 (or, fp8,
-    v_mfma_f32_32x32x64_f8f6f4 on e4m3) on register operands (tk_probe_mfma), timed with events, with amd-smi's power
-    and clocks under it.  The published peaks assume 2.4 GHz; this is the ceiling a GEMM of that class can be held
-    against on this machine."""
+def mfma_sustained_probe(device, kind=0):
+    """MFMA rate the board sustains under its power cap: a kernel of nothing but MFMA instructions on register operands
+    (tk_probe_mfma; kind 0 = v_mfma_f32_32x32x16_bf16, 1 = v_mfma_f32_32x32x64_f8f6f4 on e4m3, 2 =
+    v_mfma_f32_16x16x32_bf16), timed with events, with amd-smi's power and clocks under it.  The published peaks
+    assume 2.4 GHz; this is the ceiling a GEMM of that class can be held against on this machine."""
     from triton_amd import _native as nt
     n_wg = 2 * torch.cuda.get_device_properties(device).multi_processor_count
-    iters = 2000 if fp8 else 4000
+    iters = 2000 if kind == 1 else 4000
+    per_iter = {0: 8 * 32768.0, 1: 8 * 131072.0, 2: 16 * 16384.0}[kind]
     out = torch.zeros(n_wg * 256, dtype=torch.float32, device=device)
 
     def fn():
         with nt.on_device(device):
-            nt.check(nt.lib().tk_probe_mfma(out.data_ptr(), n_wg, iters, int(fp8), nt.stream_ptr(device)))
+            nt.check(nt.lib().tk_probe_mfma(out.data_ptr(), n_wg, iters, kind, nt.stream_ptr(device)))
 
     spin_up(fn, 0.5)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -173,8 +174,8 @@ def mfma_sustained_probe(device, fp8=False):
     e1.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / 20
-    flops = n_wg * 4 * iters * 8 * (131072.0 if fp8 else 32768.0)
-    peak = 5000.0 if fp8 else PEAK_BF16_TFLOPS
+    flops = n_wg * 4 * iters * per_iter
+    peak = 5000.0 if kind == 1 else PEAK_BF16_TFLOPS
     return dict(TFLOPs=round(flops / ms / 1e9, 1), frac_of_published_peak=round(flops / ms / 1e9 / peak, 4),
                 board=board_state_under(fn))
 
@@ -370,7 +371,7 @@ def bench_fp8(device, steps, warmup):
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
     return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8",
                 frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), board_under_step=board,
-                mfma_sustained_probe=mfma_sustained_probe(device, fp8=True))
+                mfma_sustained_probe=mfma_sustained_probe(device, kind=1))
 
 
 def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
@@ -515,7 +516,8 @@ def main():
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": GEMM1_TRAFFIC_BYTES,
                      "kernel": "moe_gemm_mxn_kernel (gather-GEMM, tiled MXFP4 W1, bias, swiglu)", "kernel_ms": round(gemm1_ms, 4),
                      "board_under_kernel": board,
-                     "mfma_sustained_probe": None if args.no_board_state else mfma_sustained_probe(device)},
+                     "mfma_sustained_probe": None if args.no_board_state else mfma_sustained_probe(device),
+                     "mfma_sustained_probe_16x16x32": None if args.no_board_state else mfma_sustained_probe(device, kind=2)},
     }
     # layer-level roofline: t_roof = max(flops / bf16 peak, algorithmic bytes / HBM peak)
     layer_bytes = 2.19e9

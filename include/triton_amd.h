@@ -395,12 +395,12 @@ int32_t tk_reduce_mid_backward(const void* dy, int32_t dtype, int64_t A, int64_t
 
 /*
  * Measurement aid (no counterpart in the reference): a kernel of nothing but MFMA instructions on register operands,
- * `n_workgroups` workgroups of four waves, `iters` x 8 instructions per wave: v_mfma_f32_32x32x16_bf16 (32768 FLOP each)
- * or, with `fp8` != 0, v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP each).  bench.py times it to report the
- * MFMA rates this board sustains under its power cap.  `out`: at least n_workgroups * 256 floats of device memory
- * (practically never written).
+ * `n_workgroups` workgroups of four waves.  `kind` 0: `iters` x 8 v_mfma_f32_32x32x16_bf16 per wave (32768 FLOP each);
+ * 1: `iters` x 8 v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP each); 2: `iters` x 16
+ * v_mfma_f32_16x16x32_bf16 (16384 FLOP each).  bench.py times it to report the MFMA rates this board sustains under
+ * its power cap.  `out`: at least n_workgroups * 256 floats of device memory (practically never written).
  */
-int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t fp8, tk_stream_t stream);
+int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t kind, tk_stream_t stream);
 
 /*
  * Per-row dynamic quantisation of bf16 activations to OCP e4m3: scales[m] = amax_m / 448 (1 for a zero

@@ -158,11 +158,13 @@ int grid_for(int64_t total) {
 // or two waves per SIMD.  Its rate under the board's power cap is the ceiling a GEMM of that MFMA class can be compared
 // with on this machine (the published peaks assume the 2.4 GHz engine clock, which the cap does not sustain under MFMA
 // load).  Operands are lane-dependent, finite and of mixed sign so that the multipliers toggle as they do on real data.
-// FP8 = false: v_mfma_f32_32x32x16_bf16 (32768 FLOP); true: v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP).
+// KIND 0: v_mfma_f32_32x32x16_bf16 (32768 FLOP); 1: v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands (131072 FLOP);
+// 2: v_mfma_f32_16x16x32_bf16 (16384 FLOP, sixteen accumulators per wave so that the pipe stays full).
 typedef int i32x8_probe_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_probe __attribute__((ext_vector_type(4)));
-template <bool FP8>
+template <int KIND>
 __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters) {
+  constexpr bool FP8 = KIND == 1;
   uint32_t raw[4][8];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -177,6 +179,24 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters) 
   for (int j = 0; j < 8; ++j)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+  if constexpr (KIND == 2) {
+    typedef float f32x4_probe __attribute__((ext_vector_type(4)));
+    f32x4_probe acc4[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc4[j] = f32x4_probe{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const u32x4_probe a = {raw[j & 3][0], raw[j & 3][1], raw[j & 3][2], raw[j & 3][3]};
+        const u32x4_probe b = {raw[(j >> 2) & 3][4], raw[(j >> 2) & 3][5], raw[(j >> 2) & 3][6], raw[(j >> 2) & 3][7]};
+        acc4[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc4[j], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[j & 7][e] += acc4[j][e];
+  } else
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -207,13 +227,15 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters) 
 
 using namespace tk;
 
-extern "C" int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t fp8, tk_stream_t stream) {
-  if (!out || n_workgroups <= 0 || iters <= 0) return fail(TK_ERR_INVALID, "tk_probe_mfma: bad arguments");
+extern "C" int32_t tk_probe_mfma(float* out, int32_t n_workgroups, int32_t iters, int32_t kind, tk_stream_t stream) {
+  if (!out || n_workgroups <= 0 || iters <= 0 || kind < 0 || kind > 2) return fail(TK_ERR_INVALID, "tk_probe_mfma: bad arguments");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (fp8)
-    hipLaunchKernelGGL(probe_mfma_kernel<true>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
+  if (kind == 1)
+    hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
+  else if (kind == 2)
+    hipLaunchKernelGGL(probe_mfma_kernel<2>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
   else
-    hipLaunchKernelGGL(probe_mfma_kernel<false>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
+    hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3((unsigned)n_workgroups), dim3(256), 0, s, out, iters);
   return check_launch("probe_mfma_kernel");
 }
 
