@@ -1,0 +1,469 @@
+// Pieces shared by the expert-GEMM kernels of this library (one translation unit per kernel family, so that they
+// compile side by side): the kernel parameter block, the tile claimer of the persistent kernels, MFMA fragment
+// traits, the shared epilogue and the launch helpers.  `tk_moe_gemm` (moe_gemm.hip) validates a descriptor, fills a
+// GemmParams and calls one family's `gemm_launch_*`.
+#pragma once
+#include <atomic>
+#include <mutex>
+#include <type_traits>
+#include <unordered_map>
+
+#include "common.h"
+#include "mx_math.h"
+
+namespace tk {
+
+enum { WK_BF16 = 0, WK_MXFP4 = 1, WK_FP8 = 2, WK_F16 = 3 };  // weight storage: bf16, packed e2m1 + e8m0 scales, e4m3, fp16 (with fp16 activations)
+
+struct GemmParams {
+  const uint8_t* x;    // bf16 or e4m3 rows
+  int32_t x_is_fp8;
+  int64_t x_stride_m;
+  const float* x_row_scale;
+  const uint8_t* w;
+  int64_t w_stride_e;  // bytes
+  int64_t w_stride_n;  // bytes
+  const uint8_t* w_scale;
+  int64_t ws_stride_e;
+  int64_t ws_stride_n;
+  const float* w_col_scale;
+  int64_t wcs_stride_e;
+  const void* bias;
+  int64_t bias_stride_e;
+  int32_t bias_is_f32;
+  const int32_t* gather;
+  const int32_t* scatter;
+  int32_t scatter_len;
+  const void* gammas;
+  int32_t gammas_is_f32;
+  const int32_t* slice_sizes;
+  const int32_t* slice_offs;
+  const int32_t* block_offs;
+  const int32_t* block_sched;
+  int32_t n_slices;
+  int32_t M, N, K;
+  uint16_t* y;
+  int64_t y_stride_m;
+  int32_t grid_n;
+  float alpha, limit;
+  int32_t has_limit;
+  int32_t y_vec;     // output rows allow 16-byte vector stores
+  int32_t bias_vec;  // bias rows allow 16-byte vector loads
+  int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
+  int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
+  int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
+  int32_t* tile_counters;  // persistent kernels: 16 zeroed words for dynamic tile claiming (9 are used), or null
+  uint32_t y_bytes;        // persistent MXFP4 kernels: bytes of the output buffer that rows may be written to (< 2 GiB)
+  int32_t combine_k;          // decode kernel: > 0 = sum the k rows of every token into combine_out (fused top-k combine)
+  uint16_t* combine_out;      // bf16 [tokens, N]
+  int64_t combine_stride;
+  int32_t* combine_counters;  // zeroed [tokens * ceil(N / 32)] words, left zero
+  const uint8_t* x_mx_scale;  // e8m0 block scales of MXFP8 activations [rows, K/32], or null
+  int64_t xs_stride_m;
+  uint8_t* y_mx_scale;        // e8m0 block scales of an MXFP8 output [rows, N_out/32], or null
+  int64_t ys_stride_m;
+};
+
+// one entry per kernel family; each returns a TK_* status
+int32_t gemm_launch_strided(const GemmParams& p, int wk, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_mxn(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_mxd(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_f8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_mx8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, bool mx_out, hipStream_t st);
+
+// Slices (experts) whose row and block offsets the persistent MXFP4 prefill kernel keeps in LDS: a tile's coordinates
+// then cost LDS reads instead of a chain of dependent global loads.  The host refuses more slices than this.
+constexpr int kMetaSlices = 1024;
+
+namespace {
+
+template <int I>
+using template_int = std::integral_constant<int, I>;
+
+// f(integral_constant<int, I>) for I in [B, E), fully expanded at compile time
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+// byte offset that a buffer resource drops (stores) or reads as zero (loads): buffers span less than 2 GiB (host check)
+constexpr uint32_t kDroppedStore = 0x80000000u;
+typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
+
+
+
+// Persistent kernels hand out tiles either statically (round r gives workgroup b tile r * grid + remap(b)) or, when the
+// caller supplies `tile_counters`, dynamically: the tile list is cut into 8 contiguous queues, one per XCD, and a
+// workgroup claims the next tile of its XCD's queue with an atomic increment (tiles that share weights or
+// activations keep running next to each other under one L2); when its queue is empty it takes from the other
+// queues in ring order.  Tiles cost different amounts (4 or 5 row fragments, partly filled column tiles), so a
+// static deal waits for the slowest tile of every round.  The claim for the NEXT tile is issued when a tile starts and
+// read when it ends, so the atomic's latency is hidden behind the tile's K loop.  Words 0..7 = next index of each
+// queue, word 8 = workgroups that have finished; the last one to finish clears all nine words, so the counters
+// are zero again when the kernel ends (launches that share the words must not overlap in time).
+
+struct TileClaimer {
+  int32_t* ctr;
+  int live;
+  int myq;
+  int pending;   // thread 0: index returned by the claim in flight
+  __device__ __forceinline__ int qbeg(int q) const { return (int)(((int64_t)live * q) >> 3); }
+  // Workgroups that start on queue q number ((grid - q + 7) / 8); each takes two tiles of the queue without asking
+  // (indices blockIdx.x / 8 and that plus their number), so the counters count from twice their number.
+  __device__ __forceinline__ int qwgs(int q) const { return ((int)gridDim.x - q + 7) >> 3; }
+  __device__ __forceinline__ int qfirst(int q) const { return 2 * qwgs(q); }
+  // second tile of this workgroup (thread-uniform, no memory access), -1 if its queue is shorter than that
+  __device__ __forceinline__ int second() const {
+    const int t = qbeg(myq) + (int)(blockIdx.x >> 3) + qwgs(myq);
+    return t < qbeg(myq + 1) ? t : -1;
+  }
+  // first tile of this workgroup (thread-uniform, no memory access), -1 if its queue is shorter than that
+  __device__ __forceinline__ int init(int32_t* c, int live_tiles) {
+    ctr = c;
+    live = live_tiles;
+    myq = blockIdx.x & 7;
+    pending = 0;
+    const int t = qbeg(myq) + (int)(blockIdx.x >> 3);
+    return t < qbeg(myq + 1) ? t : -1;
+  }
+  // thread 0: start the claim of this workgroup's next tile (own queue)
+  // (the result goes through a variable that is undefined in the other lanes: merging it with the previous value
+  // would make every lane wait for the atomic to return right here)
+  __device__ __forceinline__ void issue() {
+    int fresh;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wsometimes-uninitialized"
+    if (threadIdx.x == 0) fresh = atomicAdd(&ctr[myq], 1);
+    pending = fresh;
+#pragma clang diagnostic pop
+  }
+  // thread 0: tile id of the claim in flight, or of another queue when the own one is exhausted; -1 = no tile left.
+  // The other queues' counters are read together first, so a workgroup that finds everything taken pays two
+  // memory round trips, not eight.
+  __device__ __forceinline__ int resolve() {
+    int t = qbeg(myq) + qfirst(myq) + pending;
+    if (t < qbeg(myq + 1)) return t;
+    int seen[8];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) seen[i] = __hip_atomic_load(&ctr[(myq + i) & 7], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      const int q = (myq + i) & 7;
+      if (qbeg(q) + qfirst(q) + seen[i] >= qbeg(q + 1)) continue;  // counters only grow: taken stays taken
+      t = qbeg(q) + qfirst(q) + atomicAdd(&ctr[q], 1);
+      if (t < qbeg(q + 1)) return t;
+    }
+    return -1;
+  }
+  // thread 0, once, after the workgroup's last claim: count it as finished; the last workgroup clears the counters
+  __device__ __forceinline__ void finish() {
+    if (threadIdx.x == 0) {
+      __threadfence();
+      if (atomicAdd(&ctr[8], 1) == (int)gridDim.x - 1) {
+        __threadfence();
+        for (int i = 0; i < 9; ++i) atomicExch(&ctr[i], 0);
+      }
+    }
+  }
+};
+
+__device__ inline int xcd_remap(int pid, int total) {
+  // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2); renumber so that
+  // consecutive tile ids run on the same XCD.
+  const int per = total / 8, extra = total % 8;
+  const int grp = pid % 8, local = pid / 8;
+  return grp * per + (grp < extra ? grp : extra) + local;
+}
+
+__device__ inline float load_scalar(const void* p, int64_t i, int is_f32) {
+  return is_f32 ? static_cast<const float*>(p)[i] : bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+}
+
+// 8 e2m1 values (one dword, even element in the low nibble) -> 8 bf16 scaled by `scale`.
+__device__ inline bf16x8_t dequant8(uint32_t raw, float scale) {
+  bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(raw, scale, 0);
+  bf16x2_t b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(raw, scale, 1);
+  bf16x2_t c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(raw, scale, 2);
+  bf16x2_t d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(raw, scale, 3);
+  bf16x8_t r = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+  return r;
+}
+
+// s * (linear + 1), s = gate * sigmoid(alpha * gate).  `nalpha_log2e` = -alpha * log2(e); `limit` = +inf when the
+// activation has no limit.  v_med3_f32 clamps in one instruction; exp2 and the reciprocal are the hardware
+// approximations (1 ulp each).
+__device__ __forceinline__ float swiglu_f(float gate, float lin, float nalpha_log2e, float limit) {
+  gate = __builtin_amdgcn_fmed3f(gate, -INFINITY, limit);
+  lin = __builtin_amdgcn_fmed3f(lin, -limit, limit);
+  const float s = gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(nalpha_log2e * gate));
+  return fmaf(s, lin, s);
+}
+
+// two fp32 -> packed bf16 pair (round to nearest even), low half = a
+__device__ inline uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// output conversions of the shared epilogue: bf16, or fp16 for the fp16 x fp16 kernel
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_out2(float a, float b) {
+  if constexpr (F16) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  } else {
+    return pack_bf16x2(a, b);
+  }
+}
+template <bool F16>
+__device__ __forceinline__ uint16_t cvt_out(float a) {
+  if constexpr (F16)
+    return f32_to_f16_bits(a);
+  else
+    return f32_to_bf16_bits(a);
+}
+
+// FM = 16: v_mfma_f32_16x16x32_bf16 (lane = row % 16, 4 k-groups of 32 per 128-wide sub-stage).
+// FM = 32: v_mfma_f32_32x32x16_bf16 (lane = row % 32, 2 k-groups of 64), the full-rate shape on gfx950.
+template <int FM>
+struct Frag;
+template <>
+struct Frag<16> {
+  typedef f32x4_t acc_t;
+  static constexpr int NACC = 4;
+  static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  // the same registers read as eight fp16 values
+  static __device__ __forceinline__ acc_t mma_f16(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  // accumulator register i of lane group h holds fragment row (= output column) n_of(i, h)
+  static __device__ __forceinline__ int n_of(int i, int h) { return h * 4 + i; }
+};
+template <>
+struct Frag<32> {
+  typedef f32x16_t acc_t;
+  static constexpr int NACC = 16;
+  static __device__ __forceinline__ acc_t mma(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ acc_t mma_f16(bf16x8_t a, bf16x8_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int n_of(int i, int h) { return (i >> 2) * 8 + h * 4 + (i & 3); }
+};
+
+// Epilogue shared by the GEMM kernels.  acc[f][j] is the FM x FM fragment of column fragment f (first column
+// ncol0 + f*FM) and row fragment j (tile rows (j*WM + mw)*FM ..); register i of a lane in lane group h holds
+// output column Frag::n_of(i, h) of row lr.  Order: row/column scales, bias, activation, gate weight,
+// (scattered) store.  Everything the rows and columns need from memory is fetched before the first store.
+template <int FM, int WM, int MFW, int NFW, bool SWIGLU, bool F16OUT = false>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag<FM>::acc_t (&acc)[NFW][MFW], int expert,
+                                              int off_m, int start_m, int eM, int ncol0, bool full_n, int mw, int lr, int h) {
+  typedef Frag<FM> FR;
+  const int N = p.N;
+  const int NOUT = SWIGLU ? N / 2 : N;
+  // per-row items; rows past the slice read the slice's last row (no divergent branches around the loads)
+  float gam[MFW], rsc[MFW];
+  int64_t dst[MFW];
+  bool ok[MFW];
+  int srow[MFW];
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const int row = off_m + (j * WM + mw) * FM + lr;  // row inside the slice
+    ok[j] = row < eM;
+    srow[j] = start_m + (ok[j] ? row : eM - 1);       // row in expert-sorted order
+    gam[j] = 1.0f;
+    rsc[j] = 1.0f;
+    dst[j] = srow[j];
+  }
+  if (p.gammas) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) gam[j] = load_scalar(p.gammas, srow[j], p.gammas_is_f32);
+  }
+  if (p.scatter) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) {
+      const int sr = srow[j] < p.scatter_len ? srow[j] : p.scatter_len - 1;
+      const int v = p.scatter[sr];
+      dst[j] = srow[j] < p.scatter_len ? v : -1;
+    }
+  }
+  if (p.x_row_scale) {
+    int src[MFW];
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) src[j] = p.gather ? p.gather[srow[j]] : srow[j];
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) rsc[j] = p.x_row_scale[src[j]];
+  }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) ok[j] = ok[j] && dst[j] >= 0;
+  if (p.x_row_scale || p.w_col_scale) {  // fp8-style per-row x per-column scales
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int i = 0; i < FR::NACC; ++i) {
+        const int n = ncol0 + f * FM + FR::n_of(i, h);
+        float cs = 1.0f;
+        if (p.w_col_scale && n < N) cs = p.w_col_scale[expert * p.wcs_stride_e + n];
+#pragma unroll
+        for (int j = 0; j < MFW; ++j) acc[f][j][i] *= rsc[j] * cs;
+      }
+  }
+  if (p.bias) {
+    float b4[NFW][FR::NACC / 4][4];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int q = 0; q < FR::NACC / 4; ++q) {
+        const int n0 = ncol0 + f * FM + FR::n_of(4 * q, h);  // 4 consecutive columns
+        const int64_t bo = expert * p.bias_stride_e + n0;
+        if (full_n && p.bias_vec) {
+          if (p.bias_is_f32) {
+            const float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(p.bias) + bo);
+            b4[f][q][0] = t.x, b4[f][q][1] = t.y, b4[f][q][2] = t.z, b4[f][q][3] = t.w;
+          } else {
+            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(p.bias) + bo);
+            b4[f][q][0] = bits_f32(t.x << 16), b4[f][q][1] = bits_f32(t.x & 0xFFFF0000u);
+            b4[f][q][2] = bits_f32(t.y << 16), b4[f][q][3] = bits_f32(t.y & 0xFFFF0000u);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) b4[f][q][i] = n0 + i < N ? load_scalar(p.bias, bo + i, p.bias_is_f32) : 0.f;
+        }
+      }
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int q = 0; q < FR::NACC / 4; ++q)
+#pragma unroll
+        for (int j = 0; j < MFW; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] += b4[f][q][i];
+  }
+  // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
+  // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
+  constexpr int VW = FM == 32 ? 8 : 4;
+  constexpr int NU = FR::NACC / VW;
+  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
+  const float limit = p.has_limit ? p.limit : INFINITY;
+  const bool fast = full_n && p.y_vec;  // every column of the tile exists and rows take vector stores
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    float v[NFW][NU][VW];
+    int n0[NFW][NU];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        if constexpr (FM == 32) {
+          // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint32_t lo = f32_bits(acc[f][j][8 * u + i]), hi = f32_bits(acc[f][j][8 * u + 4 + i]);
+            auto r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo's upper half <-> hi's lower half
+            v[f][u][i] = bits_f32(r[0]);
+            v[f][u][4 + i] = bits_f32(r[1]);
+          }
+          n0[f][u] = ncol0 + f * FM + 16 * u + 8 * h;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[f][u][i] = acc[f][j][4 * u + i];
+          n0[f][u] = ncol0 + f * FM + FR::n_of(4 * u, h);
+        }
+      }
+    if (!ok[j]) continue;  // one divergent region per row fragment
+    uint16_t* yrow = p.y + dst[j] * p.y_stride_m;
+    const float g = gam[j];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        if (SWIGLU) {
+          float r[VW / 2];
+#pragma unroll
+          for (int i = 0; i < VW / 2; ++i) r[i] = swiglu_f(v[f][u][2 * i], v[f][u][2 * i + 1], nalpha_log2e, limit) * g;
+          const int o0 = n0[f][u] / 2;
+          if (fast) {
+            uint32_t w[VW / 4];
+#pragma unroll
+            for (int i = 0; i < VW / 4; ++i) w[i] = pack_out2<F16OUT>(r[2 * i], r[2 * i + 1]);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint2*>(yrow + o0) = make_uint2(w[0], w[VW / 4 - 1]);
+            else
+              *reinterpret_cast<uint32_t*>(yrow + o0) = w[0];
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i)
+              if (o0 + i < NOUT) yrow[o0 + i] = cvt_out<F16OUT>(r[i]);
+          }
+        } else {
+          if (fast) {
+            uint32_t w[VW / 2];
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i) w[i] = pack_out2<F16OUT>(v[f][u][2 * i] * g, v[f][u][2 * i + 1] * g);
+            if constexpr (VW == 8)
+              *reinterpret_cast<uint4*>(yrow + n0[f][u]) = make_uint4(w[0], w[1], w[VW / 2 - 2], w[VW / 2 - 1]);
+            else
+              *reinterpret_cast<uint2*>(yrow + n0[f][u]) = make_uint2(w[0], w[1]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW; ++i)
+              if (n0[f][u] + i < N) yrow[n0[f][u] + i] = cvt_out<F16OUT>(v[f][u][i] * g);
+          }
+        }
+      }
+  }
+}
+
+// Raises a kernel's dynamic LDS limit above 64 KiB, once per (kernel, device): the table is keyed on the kernel's
+// address, so every template instantiation (the swiglu and the plain variant of one tile shape included) has an
+// entry of its own; bit d of an entry = done on device d.
+inline int32_t allow_dynamic_lds(const void* kern, int bytes) {
+  if (bytes <= 64 * 1024) return TK_OK;
+  static std::mutex mu;
+  static std::unordered_map<const void*, uint64_t> done;
+  int dev = 0;
+  const bool known = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64;
+  if (known) {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = done.find(kern);
+    if (it != done.end() && (it->second >> dev & 1ull)) return TK_OK;
+  }
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(TK_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
+  if (known) {
+    std::lock_guard<std::mutex> lock(mu);
+    done[kern] |= 1ull << dev;
+  }
+  return TK_OK;
+}
+
+// compute units of the current device (cached per device id; racing first calls store the same value)
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+// compute units a persistent grid may fill when `idle` of them are to stay free (at least one is used)
+inline int busy_cu_count(int idle) {
+  const int n = device_cu_count() - (idle > 0 ? idle : 0);
+  return n > 0 ? n : 1;
+}
+
+}  // namespace
+}  // namespace tk
