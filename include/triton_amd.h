@@ -163,9 +163,16 @@ int32_t tk_route(const tk_route_desc* desc, tk_stream_t stream);
  * refused with TK_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on one GPU
  * (different streams, different threads) race and must be serialised by the caller; calls in stream order are
  * safe, the array's previous contents are never read.
+ * The array's device address is looked up once per device (hipGetSymbolAddress, which may load the code object):
+ * by tk_route_static_prepare(), or else by the first tk_route_static call on that device.  That lookup must not
+ * happen while a stream is capturing, so code that captures tk_route_static calls tk_route_static_prepare() (or
+ * makes one eager tk_route_static call) on each device beforehand.  Device ids 0..63 are served; others are
+ * refused with TK_ERR_UNSUPPORTED.
  */
 #define TK_ROUTE_STATIC_SCRATCH_BYTES (2 * 1024 * 1024)
 int32_t tk_route_static(const tk_route_desc* desc, tk_stream_t stream);
+/* Set-up of tk_route_static on the current device (no device work, allocates nothing; safe to call repeatedly). */
+int32_t tk_route_static_prepare(void);
 
 /*
  * Replaces `_topk_backward` (tk/topk_details/_topk_backward.py:5-51, launched by tk/topk.py:76-85): gradient of the
@@ -297,7 +304,8 @@ typedef struct tk_gemm_desc {
    * words.  NULL = fixed schedule.  No counterpart in the reference (its AMD path is not persistent). */
   int32_t* tile_counters;
   /* rows of x (with gather_indx: every index is below it); 0 = not stated (then M when not gathering).  The kernels
-   * for tiled MXFP4 weights at block_m >= 64 need x to span less than 4 GiB and refuse larger ones. */
+   * for tiled MXFP4 weights at block_m >= 64 need x to span less than 4 GiB and refuse larger ones; with
+   * gather_indx they refuse a descriptor that leaves x_rows at 0 (TK_ERR_INVALID). */
   int64_t x_rows;
   /* MXFP8 activations (x_dtype TK_E4M3): e8m0 block scales uint8 [rows of x, K / 32], unit stride along K, one per
    * 32 consecutive k of a row (tk/matmul.py:130-132 `a_mx_scale`); NULL = x is not MX-quantised.  Goes with tiled
@@ -315,8 +323,13 @@ typedef struct tk_gemm_desc {
    * scatter_indx maps expert-sorted row r to flat position t * combine_k + j; besides y [tokens * combine_k, N] the
    * kernel writes combine_out[t, :] = sum over j of y[t * combine_k + j, :] (fp32 sum in j order, bf16 result: what
    * tk_reduce_mid computes from y), by the wave that completes token t's rows last.  combine_counters:
-   * tokens * ceil(N / 32) zeroed int32 words, left zero.  A token with fewer than combine_k routed rows never
-   * completes and its row of combine_out is not written.  0 = no combine.  Replaces the separate
+   * tokens * ceil(N / 32) zeroed int32 words; a launch leaves them zero again PROVIDED every token has exactly
+   * combine_k routed rows.  A token with fewer (dropped entries, rows of experts that live on another rank) never
+   * completes: its row of combine_out is not written and its counter words stay non-zero, which corrupts that
+   * token in every later launch that shares the words, so callers must not request the combine for such routing
+   * (or must clear the words themselves, with a fill kernel on the same stream).  The Python host keeps one buffer
+   * of 65536 words per (device, stream) and falls back to the separate tk_reduce_mid launch when
+   * tokens * ceil(N / 32) exceeds it (728 tokens at N = 2880).  0 = no combine.  Replaces the separate
    * `reduce(y.view(T, k, -1), dim=1)` launch of tk/reduce.py:1143-1165 after the scatter of
    * tk/matmul_details/_matmul.py:535-569. */
   int32_t combine_k;

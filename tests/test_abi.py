@@ -114,6 +114,21 @@ def test_invalid_descriptors_return_status_and_message():
     assert lib.tk_route_workspace_bytes(4096, 128) > 0
 
 
+def test_gather_without_x_rows_is_refused_by_the_prefill_tiled_kernels():
+    """The prefill kernels for tiled MXFP4 weights address x with 32-bit offsets; with a gather the extent of x cannot
+    be derived from M, so a descriptor that leaves x_rows at 0 is refused before any launch (fake, aligned pointers)."""
+    lib = nt.lib()
+    d = nt.GemmDesc()
+    d.x, d.w, d.y, d.w_mx_scale, d.gather_indx = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000
+    d.x_dtype, d.w_dtype, d.y_dtype, d.w_layout = nt.TK_BF16, nt.TK_E2M1, nt.TK_BF16, nt.TK_W_TILED
+    d.M, d.N, d.K, d.grid_m, d.block_m, d.n_slices = 256, 256, 256, 2, 128, 1
+    d.x_stride_m, d.y_stride_m = 256, 256
+    d.w_stride_e, d.ws_stride_e = 8 * 2 * 2048, 8 * 2 * 128
+    d.x_rows = 0
+    assert lib.tk_moe_gemm(ctypes.byref(d), None) == nt.TK_ERR_INVALID
+    assert "x_rows is required" in nt.last_error()
+
+
 def test_status_to_exception_mapping():
     with pytest.raises(ValueError):
         nt.check(nt.TK_ERR_INVALID, "bad")

@@ -116,6 +116,35 @@ def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatt
     assert_allclose_gate(ref, got, what="y")
 
 
+@pytest.mark.parametrize("block_m", [16, 128, 256])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_output_given_as_a_column_slice_keeps_its_neighbours(mods, device, block_m, swiglu):
+    """`c` handed in as a column slice of a wider tensor, with a column count that is not a multiple of 8: the prefill
+    kernels for tiled MXFP4 weights write whole 16-byte pieces, so the host must not let them run over the slice's
+    last column into memory that belongs to the caller."""
+    mm, sw, tensor = mods
+    g = torch.Generator().manual_seed(11 + block_m)
+    m, n, k, n_slices = 300, 396 if not swiglu else 792, 416, 10  # N_out = 396: 396 % 8 == 4
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, "mxfp4_tiled", g, device)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    n_out = n // 2 if swiglu else n
+    wide = torch.full((m, n_out + 20), float("nan"), dtype=torch.bfloat16, device=device)
+    c = wide[:, :n_out]
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(x.to(device), W["w_dev"], None, md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]), c=c,
+                      fused_activation=act)
+    assert y.data_ptr() == c.data_ptr()
+    assert bool(torch.isnan(wide[:, n_out:]).all()), "columns next to the output slice were overwritten"
+    assert not bool(torch.isnan(wide[:, :n_out]).any())
+    ref = omoe.matmul(x, W["w_cpu"], None, sizes, w_mx_scale=W["scale_cpu"])
+    if swiglu:
+        ref = omoe.swiglu(ref, 1.702, 7.0)
+    assert_close(ref, wide[:, :n_out].cpu(), maxtol=3e-2, what="y in a slice")
+
+
 @pytest.mark.parametrize("m, n, k, mode", [(16, 256, 256, "ragged"), (300, 400, 416, "ragged"), (1000, 704, 832, "ragged"),
                                            (600, 400, 416, "plain"), (5, 2880, 2880, "ragged")])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])

@@ -407,3 +407,35 @@ def test_fused_topk_combine_equals_reduce(api, device, gptoss_weights, T):
     ref, _ = _oracle_layer_on_active_experts(x, logits, k, gptoss_weights["strided"])
     assert_close(ref, got, maxtol=3e-2, what="layer output through the fused combine")
     assert_allclose_gate(ref, got, what="layer output through the fused combine", max_bad_frac=LAYER_GATE_SLACK)
+
+
+def test_dropped_entries_take_the_separate_combine_and_leave_later_calls_clean(api, device, gptoss_weights):
+    """Routing from caller-provided indices with dropped entries (-1) gives tokens fewer than k rows.  The fused
+    combine counts arrivals per token and must not run on such routing (a token that never completes would leave its
+    counter non-zero for the next launch on the stream): `matmul_ogs` then takes GEMM + `reduce`, and a following call
+    with complete routing on the same stream is still bit-equal to `reduce`."""
+    g = torch.Generator().manual_seed(9)
+    T, E, k, d = 16, 128, 4, 2880
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
+    logits = (torch.randn((T, E), generator=g) + torch.randn((E, ), generator=g) * 1.5).to(device)
+    W = gptoss_weights["tiled"]
+    pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
+    full, _, scatter = api.routing(logits, k)
+    assert full.all_rows_live
+    indx = full.expt_indx.clone()
+    drop = torch.rand((T, k), generator=g) < 0.3
+    drop[0] = torch.tensor([False, True, False, False])  # at least one token with some, not all, of its rows
+    indx[drop.to(device)] = -1
+    part, _, scatter_p = api.routing(logits, k, expt_indx=indx)
+    assert not part.all_rows_live
+    for rdata, sc in ((part, scatter_p), (full, scatter), (part, scatter_p), (full, scatter)):
+        h = api.matmul(x, W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, precision_config=pc1,
+                       fused_activation=api.act(1.702, 7.0))
+        y = api.matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=sc.dst_indx, precision_config=pc2, gammas=rdata.gate_scal)
+        want, _ = api.reduce(y.view(T, k, -1), dim=1)
+        got = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=sc, precision_config=pc2, gammas=rdata.gate_scal)
+        if rdata is full:
+            assert torch.equal(got, want), "complete routing after a call with dropped entries: fused combine differs from reduce"
+        else:  # rows of dropped entries are never written (undefined, as in the reference): compare complete tokens
+            whole = ~drop.any(dim=1)
+            assert torch.equal(got[whole.to(device)], want[whole.to(device)])

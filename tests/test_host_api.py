@@ -191,3 +191,38 @@ def test_mx_argument_checks_match_the_reference():
         downcast_to_mxfp(torch.zeros((4, 8), dtype=torch.bfloat16), torch.uint8, axis=2)
     with pytest.raises((AssertionError, ValueError)):
         downcast_to_mxfp(torch.zeros((4, 7), dtype=torch.bfloat16), torch.uint8, axis=1)
+
+
+def test_weight_relayout_cache_key_and_invalidation():
+    """The K-contiguous copy `matmul` keeps on an N-contiguous weight tensor follows in-place torch updates through the
+    version counter; writes through `.data` do not bump it (checked here), so `invalidate_weight_cache` is the
+    documented way to drop the copy after such a write.  Inference-mode tensors have no counter and must not raise."""
+    from triton_amd.matmul import _cache_key, _k_contiguous, invalidate_weight_cache
+    w = torch.randn(2, 8, 16)
+    c0 = _k_contiguous(w)
+    assert c0.stride(-2) == 1 and torch.equal(c0, w)
+    assert _k_contiguous(w) is c0  # cached
+    w.add_(1.0)  # visible to the version counter: a new copy
+    c1 = _k_contiguous(w)
+    assert c1 is not c0 and torch.equal(c1, w)
+    v = w._version
+    w.data.mul_(2.0)  # NOT visible
+    assert w._version == v and _k_contiguous(w) is c1 and not torch.equal(c1, w)
+    invalidate_weight_cache(w)
+    c2 = _k_contiguous(w)
+    assert c2 is not c1 and torch.equal(c2, w)
+    # a different storage under the same Python object (set_) changes the key as well
+    w.set_(torch.randn(2, 8, 16))
+    assert torch.equal(_k_contiguous(w), w)
+    with torch.inference_mode():
+        wi = torch.randn(2, 8, 16)
+    assert _cache_key(wi)[1] is None
+    assert torch.equal(_k_contiguous(wi), wi)
+    # already K-contiguous weights are used in place
+    wk = torch.randn(2, 16, 8).transpose(1, 2)
+    assert _k_contiguous(wk) is wk
+
+
+def test_routing_data_records_whether_every_token_has_all_its_rows():
+    from triton_amd.legacy import RoutingData
+    assert RoutingData.__dataclass_fields__["all_rows_live"].default is False

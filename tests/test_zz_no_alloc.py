@@ -61,3 +61,47 @@ def test_route_static_refuses_sizes_beyond_its_buffer(device):
     rc = nt.lib().tk_route_static(d, None)  # refused before anything is launched
     assert rc == nt.TK_ERR_UNSUPPORTED
     assert "scratch" in nt.last_error()
+
+
+def test_route_static_in_a_hip_graph_after_one_eager_call(device):
+    """The address of the built-in scratch array is looked up on the first call on a device (or by
+    `tk_route_static_prepare`), which must happen outside graph capture; afterwards the entry point can be captured.
+    The graph is replayed twice with eager routing work in between and compared with `tk_route` each time."""
+    from triton_amd import _native as nt
+    from triton_amd.tensor_details.bitmatrix import _route
+    from triton_amd.tensor_details.ragged_tensor import _alloc
+    assert nt.lib().tk_route_static_prepare() == nt.TK_OK
+    T, E, k = 64, 128, 4
+    g = torch.Generator().manual_seed(77)
+    logits = torch.randn((T, E), generator=g).to(device)
+
+    def run(static, lg):
+        vals = torch.empty((T, k), dtype=torch.float32, device=device)
+        indx = torch.empty((T, k), dtype=torch.int16, device=device)
+        bm = torch.zeros(((E + 31) // 32, (T + 31) // 32 * 32), dtype=torch.int32, device=device)
+        ragged = _alloc(E, T * k, device)
+        r = _route(lg, indx, None, E, k, apply_softmax=True, use_provided_indx=False, vals=vals, bitmatrix_data=bm.transpose(0, 1)[:T],
+                   want_meta=True, want_extras=True, ragged=ragged, static_scratch=static)
+        return dict(vals=vals, indx=indx, bitmatrix=bm, col_sum=r["col_sum"], col_sorted=r["col_sorted_indx"],
+                    row_sorted=r["row_sorted_indx"], gather=r["gather_indx"], gammas=r["gammas"], slice_offs=ragged[0],
+                    block_offs=ragged[1])
+
+    run(True, logits)  # eager call: allocations of the Python helpers are warmed up outside the capture as well
+    torch.cuda.synchronize()
+    lg = logits.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(True, lg)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = run(True, lg)
+    for rep in range(2):
+        lg.copy_(torch.randn((T, E), generator=g).to(device))  # new inputs for every replay
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = run(False, lg)
+        torch.cuda.synchronize()
+        _assert_same(ref, got, f"graph replay {rep}")

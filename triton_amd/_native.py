@@ -88,6 +88,7 @@ SIGNATURES = {
     "tk_route_workspace_bytes": (_i64, [_i32, _i32]),
     "tk_route": (_i32, [_c.POINTER(RouteDesc), _ptr]),
     "tk_route_static": (_i32, [_c.POINTER(RouteDesc), _ptr]),
+    "tk_route_static_prepare": (_i32, []),
     "tk_topk_backward": (_i32, [_ptr, _i32, _i64, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i32, _i32, _i32, _i32, _i32, _ptr, _ptr]),
     "tk_ragged_metadata": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _i64, _i32, _ptr]),
     "tk_ragged_remap": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32, _i32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),

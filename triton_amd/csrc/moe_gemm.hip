@@ -127,7 +127,9 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);
     if (d->block_m >= 64) {
       // the prefill kernels address activation rows with 32-bit byte offsets from x
-      const int64_t rows = d->x_rows > 0 ? d->x_rows : (d->gather_indx ? 0 : d->M);
+      if (d->gather_indx && d->x_rows <= 0)
+        return fail(TK_ERR_INVALID, "tk_moe_gemm: x_rows is required with gather_indx for tiled MXFP4 weights at block_m >= 64 (the kernel addresses x with 32-bit offsets and must know its extent)");
+      const int64_t rows = d->x_rows > 0 ? d->x_rows : d->M;
       if (d->x_stride_m * 2 >= (int64_t)1 << 32 || rows * d->x_stride_m * 2 > (int64_t)1 << 32)
         return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations of 4 GiB and more are not supported with tiled MXFP4 weights (%lld rows, row stride %lld)", (long long)rows, (long long)d->x_stride_m);
     }

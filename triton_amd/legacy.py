@@ -45,6 +45,9 @@ class RoutingData:
     token_indx: torch.Tensor | None = None  # [R] int32 token feeding each expert-sorted row (= src_indx // k)
     expt_indx: torch.Tensor | None = None  # [T, k] int16 selected experts, value-descending
     gate_vals: torch.Tensor | None = None  # [T, k] gate values
+    # every token has exactly k routed rows (the router chose them itself: no caller-provided indices, which may hold
+    # dropped entries, and no row mask); only then may the scatter-GEMM also sum a token's rows
+    all_rows_live: bool = False
 
 
 def routing(logits, n_expts_act, apply_softmax: bool = True, expt_indx=None, n_rows=None):
@@ -58,7 +61,8 @@ def routing(logits, n_expts_act, apply_softmax: bool = True, expt_indx=None, n_r
     md = RaggedTensorMetadata(r["col_sum"], slice_offs, block_offs, sched)
     col, row = r["col_sorted_indx"], r["row_sorted_indx"]
     rdata = RoutingData(gate_scal=r["gammas"], expt_hist=r["col_sum"], n_expts_tot=E, n_expts_act=k, expt_data=md,
-                        token_indx=r["gather_indx"], expt_indx=indx, gate_vals=vals)
+                        token_indx=r["gather_indx"], expt_indx=indx, gate_vals=vals,
+                        all_rows_live=expt_indx is None and n_rows is None)
     return rdata, GatherIndx(src_indx=col, dst_indx=row), ScatterIndx(src_indx=row, dst_indx=col)
 
 
@@ -78,8 +82,12 @@ def matmul_ogs(x, w, bias, routing_data: RoutingData | None = None, gather_indx:
             g = torch.div(gather_indx.src_indx, k, rounding_mode="trunc").to(torch.int32)
     s = scatter_indx.dst_indx if scatter_indx is not None else None
     k = routing_data.n_expts_act if (routing_data is not None and scatter_indx is not None) else None
+    # The fused combine counts a token's rows as they arrive and needs all k of them: routing with dropped entries
+    # or a row mask, and metadata remapped to a rank's own experts, go through `reduce` instead.
+    fuse = k if (k is not None and getattr(routing_data, "all_rows_live", False)
+                 and getattr(md, "remapped_from", None) is None) else None
     y = matmul(x, w, bias, md, gather_indx=g, scatter_indx=s, precision_config=precision_config, betas=betas,
-               gammas=gammas, fused_activation=fused_activation, _combine_k=k, **kwargs)
+               gammas=gammas, fused_activation=fused_activation, _combine_k=fuse, **kwargs)
     if scatter_indx is None:
         return y
     combined = getattr(y, "_tk_combined", None)

@@ -159,12 +159,44 @@ def _strided_scale_data(scale) -> torch.Tensor:
     return scale
 
 
+def _cache_key(t: torch.Tensor):
+    """What a cached re-layout of `t` is valid for: the storage address and the version counter.  The counter misses
+    writes that bypass autograd's bookkeeping (`t.data.add_`, a kernel or collective writing through the raw
+    pointer, a DLPack consumer): after such a write call `invalidate_weight_cache(t)`.  Tensors made under
+    `torch.inference_mode` have no counter; they are keyed by address alone."""
+    try:
+        version = t._version
+    except RuntimeError:
+        version = None
+    return (t.data_ptr(), version)
+
+
+def invalidate_weight_cache(*tensors) -> None:
+    """Drops the converted copies `matmul` keeps on weight tensors (the K-contiguous re-layout of N-contiguous bf16 /
+    fp16 / fp8 weights, the 16-bit expansion of fp8 / MXFP8 weights, the converted scale layout of a `Tensor`
+    wrapper).  Needed after the weights were changed in a way their version counter does not see: `w.data.add_()`,
+    `w.data.copy_()`, an optimizer that updates `.data`, a checkpoint load or collective that writes through the raw
+    pointer.  In-place torch operations on the tensor itself (`w.add_()`, `w.copy_()`) invalidate on their own."""
+    for t in tensors:
+        if t is None:
+            continue
+        for obj in (t, getattr(getattr(t, "storage", None), "data", None)):
+            if obj is None:
+                continue
+            for name in ("_tk_k_contiguous", "_tk_expanded", "_tk_converted"):
+                if hasattr(obj, name):
+                    try:
+                        delattr(obj, name)
+                    except AttributeError:
+                        pass
+
+
 def _expanded_weights(w: torch.Tensor, scale, target: torch.dtype) -> torch.Tensor:
     """fp8 weights (with or without e8m0 scales along K) as a 16-bit float tensor, converted by the MX dequantiser ONCE
-    and kept on the weight tensor (keyed by the version counters of values and scales)."""
+    and kept on the weight tensor (keyed as `_cache_key` says, for values and scales; `invalidate_weight_cache`)."""
     from .numerics_details.mxfp import upcast_from_mxfp
     sd = _strided_scale_data(scale) if scale is not None else None
-    key = (w._version, None if sd is None else (sd.data_ptr(), sd._version), target)
+    key = (_cache_key(w), None if sd is None else _cache_key(sd), target)
     cached = getattr(w, "_tk_expanded", None)
     if cached is not None and cached[0] == key:
         return cached[1]
@@ -230,18 +262,21 @@ def _expand_operands(a, b, precision_config):
 
 def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
     """[E, K, N] weights with unit stride along K (each output column contiguous in memory).  Weights that arrive
-    N-contiguous (a plain torch [E, K, N] tensor) are re-laid out ONCE: the copy is kept on the tensor object,
-    keyed by the tensor's version counter so that an in-place update of the weights makes a new copy.  The copy
-    doubles the memory of such weights; callers that mind convert them up front (`w.transpose(-1, -2).contiguous()
-    .transpose(-1, -2)`, or `convert_layout(w, StridedLayout(-2))`) and drop the original."""
+    N-contiguous (a plain torch [E, K, N] tensor) are re-laid out ONCE: the copy is kept on the tensor object, keyed
+    by the tensor's storage address and version counter, so that an in-place torch update of the weights makes a new
+    copy.  Writes that the version counter does not see (`w.data.add_()`, raw-pointer writes) need
+    `invalidate_weight_cache(w)`.  The copy doubles the memory of such weights; callers that mind convert them up
+    front (`w.transpose(-1, -2).contiguous().transpose(-1, -2)`, or `convert_layout(w, StridedLayout(-2))`) and
+    drop the original."""
     if w.stride(-2) == 1 and (w.shape[-2] == 1 or w.stride(-1) >= w.shape[-2]):
         return w
+    key = _cache_key(w)
     cached = getattr(w, "_tk_k_contiguous", None)
-    if cached is not None and cached[0] == w._version:
+    if cached is not None and cached[0] == key:
         return cached[1]
     conv = w.transpose(-1, -2).contiguous().transpose(-1, -2)
     try:
-        w._tk_k_contiguous = (w._version, conv)
+        w._tk_k_contiguous = (key, conv)
     except (AttributeError, RuntimeError):
         pass  # a tensor subclass without a __dict__: converted per call
     return conv
@@ -421,7 +456,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
 
     `_combine_k` (used by `legacy.matmul_ogs`, not part of the reference's signature): with `scatter_indx` mapping rows
     to flat positions t * k + j, the decode kernel may also sum the k rows of every token; the result is then attached to
-    the returned tensor as `._tk_combined` ([tokens, N]) and the caller skips its `reduce`.
+    the returned tensor as `._tk_combined` ([tokens, N]) and the caller skips its `reduce`.  The caller vouches that
+    EVERY token has exactly k routed rows: a token with fewer leaves its arrival counter non-zero for the next launch.
     """
     if b_ragged_metadata is not None:
         return _matmul_ragged_k(a, b, bias, a_ragged_metadata, b_ragged_metadata, gather_indx, scatter_indx, precision_config,
@@ -518,6 +554,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     assert K == K_W, f"reduction dims differ: a has K={K}, b has K={K_W}"
     is_ragged = a_ragged_metadata is not None
     if is_ragged and getattr(a_ragged_metadata, "remapped_from", None) is not None:
+        _combine_k = None  # only the local experts' rows arrive: tokens are incomplete
         a_ragged_metadata = _localise_remapped_metadata(a_ragged_metadata, w.shape[0], M)
     n_slices = a_ragged_metadata.n_slices if is_ragged else w.shape[0]
     if not is_ragged and w.shape[0] != 1:
@@ -557,6 +594,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
             and c_scale.stride(-1) == 1, f"c_mx_scale must be uint8 [{y_rows}, {out_shape[1] // MXFP_BLOCK_SIZE}]"
         precision_config.c_microblock_size = MXFP_BLOCK_SIZE
         precision_config.c_value_pack_factor = 1
+    caller_c = c is not None
     if c is None:
         c = torch.empty(out_shape, dtype=out_dtype, device=a.device)
     else:
@@ -705,9 +743,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     y_buf = c
     if tiled and block_m >= 64 and not mx_act:
         # the prefill kernels write whole 16-byte pieces through a buffer resource: rows 16-byte aligned and padded to
-        # a multiple of 8 columns; an output that is not goes through a padded buffer and is copied
+        # a multiple of 8 columns; an output that is not goes through a padded buffer and is copied.  So does a
+        # caller's own `c` whose last piece would spill past its columns (they may belong to a wider tensor).
         n_pad = (out_shape[1] + 7) // 8 * 8
-        if c.stride(0) % 8 or c.data_ptr() % 16 or c.stride(0) < n_pad:
+        if c.stride(0) % 8 or c.data_ptr() % 16 or c.stride(0) < n_pad or (caller_c and out_shape[1] % 8):
             y_buf = torch.empty((out_shape[0], n_pad), dtype=c.dtype, device=c.device)[:, :out_shape[1]]
     d.y = y_buf.data_ptr()
     d.y_dtype = nt.TORCH_TO_TK[c.dtype]
