@@ -374,6 +374,70 @@ typedef struct tk_ragged_k_desc {
 
 int32_t tk_ragged_k_gemm(const tk_ragged_k_desc* desc, tk_stream_t stream);
 
+/*
+ * A whole decode-sized MoE FFN layer in ONE launch:
+ *   out[t, :] = sum over j < k of gate[t, j] * ( swiglu( x[t, :] @ W1[e] + b1[e] ) @ W2[e] + b2[e] ),  e = indx[t, j]
+ * with (indx, gate) = top-k (+softmax) of logits[t, :] exactly as tk_route selects them.  Replaces, for
+ * n_tokens * k <= TK_DECODE_MAX_ROWS, the sequence the reference's MoE block issues (python/triton_kernels/bench/
+ * bench_mlp.py:72-79 and tests/test_distributed.py:203-220): `topk` + metadata launches (tk/topk.py:59-67,
+ * tk/tensor_details/bitmatrix.py:128-145, tk/tensor_details/ragged_tensor.py:197-208), two `_matmul` launches
+ * (tk/matmul.py:659-726: gather + fused swiglu, then scatter + gammas) and `reduce` over the k rows of a token
+ * (tk/reduce.py:1143-1165).  Same arithmetic as that sequence on this library's kernels: bf16 MFMA with fp32
+ * accumulation on MXFP4 weights expanded in registers, swiglu on the fp32 accumulator, the hidden activations and the
+ * k partial rows rounded to bf16, the combine summed in fp32 in j order.
+ *
+ * W1 [E, d_model, 2*d_ff] and W2 [E, d_ff, d_model] are MXFP4 in the tiled layout (TK_W_TILED) with tiled scales;
+ * x is bf16 [n_tokens, d_model]; biases bf16 or fp32 [E, N] or NULL; out bf16 [n_tokens, d_model].
+ * Limits: n_tokens * k <= TK_DECODE_MAX_ROWS, n_experts <= TK_DECODE_MAX_EXPERTS, d_model and d_ff <= 3072 and
+ * multiples of 8; otherwise TK_ERR_UNSUPPORTED (callers then take tk_route + tk_moe_gemm).
+ *
+ * The kernel is persistent: its workgroups must all be resident together (the grid is sized from the occupancy the
+ * runtime reports) because workgroups of the second GEMM wait for the first GEMM's rows of other workgroups.  Two
+ * launches of it that overlap in time on one device (different streams) could each hold part of the GPU and wait
+ * for the rest; callers serialise them.  Every wait is bounded by `spin_limit` polls (0 = default, about a second):
+ * a wait that runs out sets bit 0 of the error word and the launch finishes with a wrong result instead of hanging.
+ *
+ * workspace: tk_moe_decode_layer_workspace_bytes(...) bytes, 256-byte aligned: the hidden activations, the k partial
+ * rows and, at its end, the synchronisation words: [0] finished workgroups, [1] error word (sticky; 0 = fine),
+ * then the counters.  The words must be ZERO before the first launch; a launch leaves them zero (except a raised
+ * error word), so launches in stream order share one workspace.  indx_out / vals_out: optional [n_tokens, k]
+ * int16 / fp32 copies of the routing decision.
+ */
+#define TK_DECODE_MAX_ROWS 256
+#define TK_DECODE_MAX_EXPERTS 512
+typedef struct tk_decode_layer_desc {
+  const void* x; /* bf16 [n_tokens, d_model], unit stride along d_model */
+  int64_t x_stride_m;
+  const void* logits; /* [n_tokens, n_experts], TK_F32 or TK_BF16 */
+  int32_t logits_dtype;
+  int64_t logits_stride_m;
+  int32_t n_tokens, n_experts, k, apply_softmax;
+  int32_t d_model, d_ff;
+  const void* w1; /* tiled MXFP4 [E, d_model, 2*d_ff] */
+  const void* w1_mx_scale;
+  int64_t w1_stride_e, w1s_stride_e; /* bytes */
+  const void* b1;                    /* [E, 2*d_ff] or NULL */
+  int32_t b1_dtype;
+  int64_t b1_stride_e;
+  const void* w2; /* tiled MXFP4 [E, d_ff, d_model] */
+  const void* w2_mx_scale;
+  int64_t w2_stride_e, w2s_stride_e;
+  const void* b2; /* [E, d_model] or NULL */
+  int32_t b2_dtype;
+  int64_t b2_stride_e;
+  float act_alpha, act_limit; /* swiglu */
+  int32_t act_has_limit;
+  void* out; /* bf16 [n_tokens, d_model] */
+  int64_t out_stride_m;
+  void* indx_out;   /* optional int16 [n_tokens, k] */
+  float* vals_out;  /* optional fp32 [n_tokens, k] */
+  void* workspace;
+  int32_t spin_limit;
+} tk_decode_layer_desc;
+
+int64_t tk_moe_decode_layer_workspace_bytes(int32_t n_tokens, int32_t k, int32_t n_experts, int32_t d_ff, int32_t d_model);
+int32_t tk_moe_decode_layer(const tk_decode_layer_desc* desc, tk_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Element-wise companions of the GEMM
  * ---------------------------------------------------------------------------------------------- */

@@ -65,19 +65,21 @@ def test_struct_field_order_matches_header():
     assert _declared_struct_fields("tk_route_desc") == [f[0] for f in nt.RouteDesc._fields_]
     assert _declared_struct_fields("tk_gemm_desc") == [f[0] for f in nt.GemmDesc._fields_]
     assert _declared_struct_fields("tk_ragged_k_desc") == [f[0] for f in nt.RaggedKDesc._fields_]
+    assert _declared_struct_fields("tk_decode_layer_desc") == [f[0] for f in nt.DecodeLayerDesc._fields_]
 
 
 def test_header_is_plain_c_and_struct_sizes_match(tmp_path):
     src = tmp_path / "probe.c"
     src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "triton_amd.h"\n'
-                   'int main(void){printf("%zu %zu %zu %zu %zu\\n", sizeof(tk_route_desc), sizeof(tk_gemm_desc),'
-                   ' offsetof(tk_gemm_desc, y), offsetof(tk_route_desc, workspace), sizeof(tk_ragged_k_desc));return 0;}\n')
+                   'int main(void){printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(tk_route_desc), sizeof(tk_gemm_desc),'
+                   ' offsetof(tk_gemm_desc, y), offsetof(tk_route_desc, workspace), sizeof(tk_ragged_k_desc),'
+                   ' sizeof(tk_decode_layer_desc), offsetof(tk_decode_layer_desc, workspace));return 0;}\n')
     exe = tmp_path / "probe"
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
                    check=True)
     sizes = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
     assert sizes == [ctypes.sizeof(nt.RouteDesc), ctypes.sizeof(nt.GemmDesc), nt.GemmDesc.y.offset, nt.RouteDesc.workspace.offset,
-                     ctypes.sizeof(nt.RaggedKDesc)]
+                     ctypes.sizeof(nt.RaggedKDesc), ctypes.sizeof(nt.DecodeLayerDesc), nt.DecodeLayerDesc.workspace.offset]
 
 
 def test_enum_values_match_header():

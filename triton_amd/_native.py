@@ -80,6 +80,20 @@ class RaggedKDesc(_c.Structure):
     ]
 
 
+class DecodeLayerDesc(_c.Structure):
+    """struct tk_decode_layer_desc (field order and types follow include/triton_amd.h)."""
+    _fields_ = [
+        ("x", _ptr), ("x_stride_m", _i64), ("logits", _ptr), ("logits_dtype", _i32), ("logits_stride_m", _i64),
+        ("n_tokens", _i32), ("n_experts", _i32), ("k", _i32), ("apply_softmax", _i32), ("d_model", _i32), ("d_ff", _i32),
+        ("w1", _ptr), ("w1_mx_scale", _ptr), ("w1_stride_e", _i64), ("w1s_stride_e", _i64),
+        ("b1", _ptr), ("b1_dtype", _i32), ("b1_stride_e", _i64),
+        ("w2", _ptr), ("w2_mx_scale", _ptr), ("w2_stride_e", _i64), ("w2s_stride_e", _i64),
+        ("b2", _ptr), ("b2_dtype", _i32), ("b2_stride_e", _i64),
+        ("act_alpha", _f32), ("act_limit", _f32), ("act_has_limit", _i32),
+        ("out", _ptr), ("out_stride_m", _i64), ("indx_out", _ptr), ("vals_out", _ptr), ("workspace", _ptr), ("spin_limit", _i32),
+    ]
+
+
 # name -> (restype, argtypes); must list every symbol include/triton_amd.h declares.
 SIGNATURES = {
     "tk_version": (_i32, []),
@@ -94,6 +108,8 @@ SIGNATURES = {
     "tk_ragged_remap": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i32, _i32, _i32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
     "tk_moe_gemm": (_i32, [_c.POINTER(GemmDesc), _ptr]),
     "tk_ragged_k_gemm": (_i32, [_c.POINTER(RaggedKDesc), _ptr]),
+    "tk_moe_decode_layer_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32, _i32]),
+    "tk_moe_decode_layer": (_i32, [_c.POINTER(DecodeLayerDesc), _ptr]),
     "tk_probe_mfma": (_i32, [_ptr, _i32, _i32, _i32, _ptr]),
     "tk_swiglu": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i64, _f32, _f32, _i32, _ptr, _ptr]),
     "tk_reduce_mid": (_i32, [_ptr, _i32, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
