@@ -248,45 +248,56 @@ def capture(fn):
     return graph, out
 
 
-def bench_decode(device, steps, warmup):
-    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched.  Three layers with
-    their own weight copies (so that no layer finds its weights in the last-level cache) are captured in ONE HIP graph,
-    as a serving loop captures a decode step over all its layers; the time of a layer is the replay time / 3.  Every
-    layer's output of every checked replay is compared with the eager result before timing."""
+def bench_decode(device, steps, warmup, n_layers=10):
+    """Config 4: T in {1, 4, 16, 64}, skewed router; GB/s on the expert weights actually touched.  `n_layers` layers
+    with their own weight copies are captured in ONE HIP graph, as a serving loop captures a decode step over all its
+    layers (gpt-oss-120b has 36); the time of a layer is the replay time / n_layers.  Ten copies rotate at least
+    530 MB of touched weights at every T (the last-level cache holds 256 MB), so no layer finds its weights cached.
+    Two paths are timed on the same inputs: `moe_mlp` (one launch per layer from 8 routed rows on) and the three-call
+    sequence routing -> matmul_ogs -> matmul_ogs.  Every layer's output of every checked replay is compared with the
+    eager result before timing."""
+    from triton_kernels.moe_decode import MIN_ROWS, moe_mlp
     E, k, d, f2 = 128, 4, 2880, 5760
-    copies = [to_matmul_layout(w) for w in make_moe_weights(E, d, f2, seed=3, device=device, n_copies=3)]
+    copies = [to_matmul_layout(w) for w in make_moe_weights(E, d, f2, seed=3, device=device, n_copies=n_layers)]
     per_expert = d * f2 // 2 + d * f2 // 32 + (f2 // 2) * d // 2 + (f2 // 2) * d // 32
     res = {}
     g = torch.Generator().manual_seed(3)
     ebias = torch.randn((E, ), generator=g) * 1.5
     layers = [MoeLayer(w, k) for w in copies]
-    n_layers = len(layers)
     for T in (1, 4, 16, 64):
         x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
         logits = (torch.randn((T, E), generator=g) + ebias).to(device)
-        eager = [layer(x, logits) for layer in layers]
-        active = int((eager[0][1].expt_hist > 0).sum())
-
-        def step_eager():
-            for layer in layers:
-                layer(x, logits)
-
-        ms_eager = time_steps(step_eager, steps, warmup) / n_layers
-        graph, outs = capture(lambda: [layer(x, logits)[0] for layer in layers])
-        for rep in range(2):  # replays with eager work in between, each compared with the eager outputs
-            graph.replay()
-            torch.cuda.synchronize()
-            for out, (ref, _) in zip(outs, eager):
-                if not torch.equal(out, ref):
-                    raise RuntimeError(f"decode T={T}: graph replay {rep} differs from the eager result")
-            step_eager()
-        ms = time_steps(graph.replay, steps, warmup) / n_layers
+        active = int((layers[0](x, logits)[1].expt_hist > 0).sum())
         gbytes = active * per_expert / 1e9
-        res[f"T{T}"] = dict(ms=round(ms, 4), ms_eager=round(ms_eager, 4), active_experts=active, weight_GB=round(gbytes, 4),
-                            GBps=round(gbytes / (ms * 1e-3), 1), frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
-        if T == 16:
-            res[f"T{T}"]["board_under_replay"] = board_state_under(graph.replay)
-        del graph
+
+        def three_call():
+            return [layer(x, logits)[0] for layer in layers]
+
+        def one_call():
+            return [moe_mlp(x, logits, k, l.W["w1"], l.W["b1"], l.W["w2"], l.W["b2"], l.pc1, l.pc2, l.act) for l in layers]
+
+        timed = {}
+        for name, fn in (("three_calls", three_call), ("moe_mlp", one_call)):
+            eager = fn()
+            ms_eager = time_steps(fn, steps, warmup) / n_layers
+            graph, outs = capture(fn)
+            for rep in range(2):  # replays with eager work in between, each compared with the eager outputs
+                graph.replay()
+                torch.cuda.synchronize()
+                for out, ref in zip(outs, eager):
+                    if not torch.equal(out, ref):
+                        raise RuntimeError(f"decode T={T} ({name}): graph replay {rep} differs from the eager result")
+                fn()
+            ms = time_steps(graph.replay, steps, warmup) / n_layers
+            timed[name] = dict(ms=round(ms, 4), ms_eager=round(ms_eager, 4), GBps=round(gbytes / (ms * 1e-3), 1),
+                               frac_hbm=round(gbytes / (ms * 1e-3) / PEAK_HBM_GBPS, 4))
+            if T == 16 and name == "moe_mlp":
+                timed[name]["board_under_replay"] = board_state_under(graph.replay)
+            del graph
+        best = min(timed, key=lambda n: timed[n]["ms"])
+        res[f"T{T}"] = dict(ms=timed[best]["ms"], path=best, launches_per_layer=1 if (best == "moe_mlp" and T * k >= MIN_ROWS) else 3,
+                            active_experts=active, weight_GB=round(gbytes, 4), GBps=timed[best]["GBps"], frac_hbm=timed[best]["frac_hbm"],
+                            layers_per_graph=n_layers, rotated_weight_GB=round(gbytes * n_layers, 3), **{n: timed[n] for n in timed})
     return res
 
 

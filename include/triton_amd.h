@@ -336,6 +336,19 @@ typedef struct tk_gemm_desc {
   void* combine_out; /* bf16 [tokens, N], unit stride along N */
   int64_t combine_stride_m;
   int32_t* combine_counters;
+  /* Less common options of the reference's epilogue, in its order (tk/matmul_details/_matmul.py:547-559,581-591):
+   *   acc = acc * scales + bias * betas[r];  acc *= out_alpha;  out = act(acc) * gammas[r];  out += acc_in[row, :]
+   * betas: per expert-sorted row, fp32 or bf16 (`betas`, tk/matmul.py:251); out_alpha: scalar, applied when
+   * has_out_alpha != 0 (tk/matmul.py:253); acc_in: a tensor of the output's shape and type that is added to the
+   * result (`c_acc_in`, tk/matmul.py:258,529-535; not together with scatter_indx).  Served by the kernels with the
+   * shared epilogue: strided weights, tiled e4m3 weights, tiled MXFP4 weights at block_m 16 / 32 without the fused
+   * combine, and MXFP8 activations without an MX output; any other combination is refused with TK_ERR_UNSUPPORTED. */
+  const void* betas;
+  int32_t betas_dtype;
+  int32_t has_out_alpha;
+  float out_alpha;
+  const void* acc_in;
+  int64_t acc_in_stride_m;
 } tk_gemm_desc;
 
 #define TK_GEMM_TILE_COUNTER_WORDS 16

@@ -32,8 +32,12 @@ def dequant_weight(w: torch.Tensor, w_mx_scale: torch.Tensor | None, w_col_scale
 
 
 def matmul(x, w, bias, slice_sizes=None, gather_indx=None, scatter_indx=None, gammas=None, betas=None,
-           w_mx_scale=None, x_row_scale=None, w_col_scale=None, out_dtype=None):
-    """Y[dst(r)] = cast(((X[src(r)] @ W[e(r)]) + bias[e(r)]*beta_r) * gamma_r)   (matmul.py:840-931).
+           w_mx_scale=None, x_row_scale=None, w_col_scale=None, out_dtype=None, out_alpha=None, acc_in=None):
+    """Y[dst(r)] = cast(((X[src(r)] @ W[e(r)]) + bias[e(r)]*beta_r) * out_alpha * gamma_r + acc_in[r])   (matmul.py:840-931).
+
+    `out_alpha` and `acc_in` are not arguments of the reference's torch twin; they follow its kernel's epilogue
+    (matmul_details/_matmul.py:547-559: `acc = acc + bias * betas; acc *= out_alpha; out = act(acc); out *= gammas`,
+    and :581-591: `out += load(OutAcc)`), and are pinned against a float64 closed form in tests/test_oracle_moe.py.
 
     `x [M,K]`; `w [E,K,N]` (or `[K,N]`); `slice_sizes [E]` rows per expert in sorted order (None: one
     slice covering every row); accumulation in fp32 via `torch.matmul`; the result is rounded to
@@ -69,8 +73,13 @@ def matmul(x, w, bias, slice_sizes=None, gather_indx=None, scatter_indx=None, ga
             b = bias.detach().to("cpu").to(torch.float32)
             b = b[e] if b.ndim == 2 else b
             acc += b if betas is None else b[None, :] * betas.to("cpu").to(torch.float32)[lo:hi, None]
+        if out_alpha is not None:
+            acc *= float(out_alpha)
         if gammas is not None:
             acc *= gammas.detach().to("cpu").to(torch.float32)[lo:hi, None]
+        if acc_in is not None:
+            assert scatter_indx is None  # matmul.py:531
+            acc += acc_in.detach().to("cpu").to(torch.float32)[lo:hi, :]
         y[lo:hi, :] = acc.to(out_dtype)
     if scatter_indx is None:
         return y

@@ -86,9 +86,12 @@ def test_config4_full_shape_one_launch(api, device, gptoss_weights, T):
     assert torch.equal(rdata.expt_indx, indx)
     assert_close(rdata.gate_vals, vals, what="gate values against tk_route")
     assert_close(three.cpu(), out, maxtol=3e-2, what="one launch against three calls")
-    # moe_mlp picks the single launch here
+    # moe_mlp picks the single launch from 8 routed rows on, the three calls below
     again = api.md.moe_mlp(xd, ld, k, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)
-    assert torch.equal(again, out), "two launches on the same inputs differ"
+    if T * k >= api.md.MIN_ROWS:
+        assert torch.equal(again, out), "two launches on the same inputs differ"
+    else:
+        assert torch.equal(again, three), "moe_mlp below its row threshold is the three-call sequence"
 
 
 def test_heavy_skew_many_row_blocks_on_one_expert(api, device, gptoss_weights):

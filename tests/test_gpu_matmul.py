@@ -116,6 +116,42 @@ def test_matmul(mods, device, m, n, k, mode, wkind, block_m, do_gather, do_scatt
     assert_allclose_gate(ref, got, what="y")
 
 
+@pytest.mark.parametrize("wkind", ["bf16", "bf16_kmajor", "mxfp4", "mxfp4_tiled"])
+@pytest.mark.parametrize("block_m", [16, 128])
+@pytest.mark.parametrize("do_gather, swiglu", [(False, False), (True, False), (False, True)])
+def test_betas_out_alpha_c_acc_in(mods, device, wkind, block_m, do_gather, swiglu):
+    """`betas` (per-row multiplier of the bias), `out_alpha` and `c_acc_in` of the reference's signature
+    (triton_kernels/matmul.py:251-258) in its epilogue order (matmul_details/_matmul.py:547-559,581-591):
+    y = act((x @ w + bias * beta) * alpha) * gamma + c_acc_in."""
+    mm, sw, tensor = mods
+    g = torch.Generator().manual_seed(77 + block_m)
+    m, n, k, n_slices = 300, 400, 416, 10
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, wkind, g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    gather = torch.randint(0, m, (m, ), generator=g, dtype=torch.int32) if do_gather else None
+    betas = torch.rand((m, ), generator=g) + 0.5
+    gammas = 2.0**torch.randint(-3, 0, (m, ), generator=g).float()
+    n_out = n // 2 if swiglu else n
+    acc_in = torch.randn((m, n_out), generator=g).to(torch.bfloat16)
+    alpha = 0.75
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    dev = lambda t: None if t is None else t.to(device)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        y = mm.matmul(x.to(device), W["w_dev"], dev(bias), md, gather_indx=dev(gather), precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]),
+                      betas=dev(betas), gammas=dev(gammas), out_alpha=alpha, c_acc_in=dev(acc_in), fused_activation=act)
+    if swiglu:  # the activation sits between out_alpha and the gate weight
+        pre = omoe.matmul(x, W["w_cpu"], bias, sizes, gather_indx=gather, betas=betas, out_alpha=alpha, w_mx_scale=W["scale_cpu"], out_dtype=torch.float32)
+        ref = (omoe.swiglu(pre, 1.702, 7.0, out_dtype=torch.float32) * gammas[:, None] + acc_in.float()).to(torch.bfloat16)
+    else:
+        ref = omoe.matmul(x, W["w_cpu"], bias, sizes, gather_indx=gather, gammas=gammas, betas=betas, out_alpha=alpha, acc_in=acc_in,
+                          w_mx_scale=W["scale_cpu"])
+    assert_close(ref, y.cpu(), maxtol=3e-2, what="y with betas / out_alpha / c_acc_in")
+    assert_allclose_gate(ref, y.cpu(), what="y with betas / out_alpha / c_acc_in")
+
+
 @pytest.mark.parametrize("block_m", [16, 128, 256])
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_output_given_as_a_column_slice_keeps_its_neighbours(mods, device, block_m, swiglu):
@@ -458,9 +494,10 @@ def test_rejected_options(mods, device):
     mm, _, _ = mods
     x = torch.zeros((4, 32), dtype=torch.bfloat16, device=device)
     w = torch.zeros((1, 32, 16), dtype=torch.bfloat16, device=device)
-    with pytest.raises(NotImplementedError):
-        mm.matmul(x, w, None, betas=torch.ones(4, device=device))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(AssertionError):  # c_acc_in + scatter (triton_kernels/matmul.py:531)
+        mm.matmul(x, w, None, c_acc_in=torch.zeros((4, 16), dtype=torch.bfloat16, device=device),
+                  scatter_indx=torch.arange(4, dtype=torch.int32, device=device))
+    with pytest.raises(NotImplementedError):  # c_acc_in of another type than the output
         mm.matmul(x, w, None, c_acc_in=torch.zeros((4, 16), device=device))
     with pytest.raises(NotImplementedError):  # NVFP4 output (float8 block scales) is a Blackwell format
         mm.matmul(x, w, None, epilogue=mm.Epilogue(mm.FnSpecs(mm.FnName.QUANTIZE_NVFP4.name, object(), (), ()), (), (), 2.0))

@@ -225,3 +225,29 @@ def test_ragged_k_is_a_masked_dense_product():
     # a transposed (strided) operand is the same problem
     got3 = omoe.matmul_ragged_k(a.t().contiguous().t(), b, sizes, a_offs, b_offs, out_dtype=torch.float32)
     assert torch.equal(got3, got)
+
+
+def test_matmul_betas_out_alpha_acc_in_against_float64():
+    """The less common epilogue options in the kernel's order (matmul_details/_matmul.py:547-559,581-591):
+    y = ((x @ w + bias * beta) * alpha) * gamma + acc_in, checked element-wise against float64 on a small ragged case;
+    a swapped order (alpha applied to the accumulated input, beta applied to the product) would miss by far more."""
+    g = torch.Generator().manual_seed(5)
+    M, K, N, E = 37, 24, 20, 3
+    sizes = torch.tensor([10, 0, 27], dtype=torch.int32)
+    x = torch.randn((M, K), generator=g)
+    w = torch.randn((E, K, N), generator=g)
+    bias = torch.randn((E, N), generator=g)
+    betas, gammas = torch.rand((M, ), generator=g) + 0.5, torch.rand((M, ), generator=g) + 0.5
+    acc_in = torch.randn((M, N), generator=g)
+    alpha = 0.37
+    got = omoe.matmul(x, w, bias, sizes, gammas=gammas, betas=betas, out_alpha=alpha, acc_in=acc_in, out_dtype=torch.float32)
+    ref = torch.zeros((M, N), dtype=torch.float64)
+    lo = 0
+    for e, n in enumerate(sizes.tolist()):
+        hi = lo + n
+        t = x[lo:hi].double() @ w[e].double() + bias[e].double()[None, :] * betas[lo:hi].double()[:, None]
+        ref[lo:hi] = t * alpha * gammas[lo:hi].double()[:, None] + acc_in[lo:hi].double()
+        lo = hi
+    assert float((got.double() - ref).abs().max()) < 1e-4
+    wrong = omoe.matmul(x, w, bias, sizes, gammas=gammas, betas=betas, out_dtype=torch.float32) + alpha * acc_in
+    assert float((wrong.double() - ref).abs().max()) > 1e-2

@@ -66,6 +66,7 @@ class GemmDesc(_c.Structure):
         ("w_layout", _i32), ("idle_cus", _i32), ("tile_counters", _ptr), ("x_rows", _i64),
         ("x_mx_scale", _ptr), ("xs_stride_m", _i64), ("y_mx_scale", _ptr), ("ys_stride_m", _i64),
         ("combine_k", _i32), ("combine_out", _ptr), ("combine_stride_m", _i64), ("combine_counters", _ptr),
+        ("betas", _ptr), ("betas_dtype", _i32), ("has_out_alpha", _i32), ("out_alpha", _f32), ("acc_in", _ptr), ("acc_in_stride_m", _i64),
     ]
 
 

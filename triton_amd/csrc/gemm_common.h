@@ -62,6 +62,13 @@ struct GemmParams {
   int64_t xs_stride_m;
   uint8_t* y_mx_scale;        // e8m0 block scales of an MXFP8 output [rows, N_out/32], or null
   int64_t ys_stride_m;
+  // options of the shared epilogue only (the host keeps them away from the kernels with an epilogue of their own)
+  const void* betas;          // per expert-sorted row multiplier of the bias, or null
+  int32_t betas_is_f32;
+  int32_t has_out_alpha;      // acc *= out_alpha behind the bias, in front of the activation
+  float out_alpha;
+  const uint16_t* acc_in;     // tensor of the output's shape and type added to the result (behind the gate weight), or null
+  int64_t acc_in_stride_m;
 };
 
 // one entry per kernel family; each returns a TK_* status
@@ -317,6 +324,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
         for (int j = 0; j < MFW; ++j) acc[f][j][i] *= rsc[j] * cs;
       }
   }
+  float beta[MFW];
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) beta[j] = 1.0f;
+  if (p.betas) {
+#pragma unroll
+    for (int j = 0; j < MFW; ++j) beta[j] = load_scalar(p.betas, srow[j], p.betas_is_f32);
+  }
   if (p.bias) {
     float b4[NFW][FR::NACC / 4][4];
 #pragma unroll
@@ -346,7 +360,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
 #pragma unroll
         for (int j = 0; j < MFW; ++j)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] += b4[f][q][i];
+          for (int i = 0; i < 4; ++i) acc[f][j][4 * q + i] = p.betas ? fmaf(b4[f][q][i], beta[j], acc[f][j][4 * q + i]) : acc[f][j][4 * q + i] + b4[f][q][i];
+  }
+  if (p.has_out_alpha) {
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int j = 0; j < MFW; ++j)
+#pragma unroll
+        for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] *= p.out_alpha;
   }
   // VW consecutive output columns per lane: 4 as the MFMA leaves them (16x16), or 8 after the two lane
   // halves of a 32x32 fragment exchange their 4-column groups (v_permlane32_swap)
@@ -382,6 +404,35 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, typename Frag
     if (!ok[j]) continue;  // one divergent region per row fragment
     uint16_t* yrow = p.y + dst[j] * p.y_stride_m;
     const float g = gam[j];
+    if (p.acc_in) {
+      // out = act(...) * gate + acc_in[row, column]: fold the gate weight in here and add, element by element (an
+      // option off the tuned paths)
+      const uint16_t* arow = p.acc_in + dst[j] * p.acc_in_stride_m;
+#pragma unroll
+      for (int f = 0; f < NFW; ++f)
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+          if (SWIGLU) {
+            const int o0 = n0[f][u] / 2;
+#pragma unroll
+            for (int i = 0; i < VW / 2; ++i) {
+              if (o0 + i < NOUT) {
+                const float a = F16OUT ? f16_bits_to_f32(arow[o0 + i]) : bf16_bits_to_f32(arow[o0 + i]);
+                yrow[o0 + i] = cvt_out<F16OUT>(swiglu_f(v[f][u][2 * i], v[f][u][2 * i + 1], nalpha_log2e, limit) * g + a);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < VW; ++i) {
+              if (n0[f][u] + i < N) {
+                const float a = F16OUT ? f16_bits_to_f32(arow[n0[f][u] + i]) : bf16_bits_to_f32(arow[n0[f][u] + i]);
+                yrow[n0[f][u] + i] = cvt_out<F16OUT>(v[f][u][i] * g + a);
+              }
+            }
+          }
+        }
+      continue;
+    }
 #pragma unroll
     for (int f = 0; f < NFW; ++f)
 #pragma unroll

@@ -87,6 +87,16 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     p.combine_stride = d->combine_stride_m;
     p.combine_counters = d->combine_counters;
   }
+  p.betas = d->betas;
+  p.betas_is_f32 = d->betas_dtype == TK_F32;
+  if (d->betas && d->betas_dtype != TK_F32 && d->betas_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: betas must be fp32 or bf16");
+  p.has_out_alpha = d->has_out_alpha != 0;
+  p.out_alpha = d->out_alpha;
+  p.acc_in = static_cast<const uint16_t*>(d->acc_in);
+  p.acc_in_stride_m = d->acc_in_stride_m;
+  const bool extras = d->betas || d->has_out_alpha || d->acc_in;
+  if (d->acc_in && d->scatter_indx) return fail(TK_ERR_INVALID, "tk_moe_gemm: acc_in is not supported together with scatter_indx");
+  if (extras && d->combine_k > 0) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: betas / out_alpha / acc_in are not supported together with the fused top-k combine");
   p.x_mx_scale = static_cast<const uint8_t*>(d->x_mx_scale);
   p.xs_stride_m = d->xs_stride_m;
   p.y_mx_scale = static_cast<uint8_t*>(d->y_mx_scale);
@@ -113,6 +123,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if ((reinterpret_cast<uintptr_t>(d->w) & 15) || d->w_stride_e % 16 || (reinterpret_cast<uintptr_t>(d->w_mx_scale) & 3) || d->ws_stride_e % 4) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: tiled weights must be 16-byte aligned");
     const int64_t nfr = cdiv(d->N, 32), nst = cdiv(d->K, 128);
     if (d->n_slices > 1 && (d->w_stride_e < nfr * nst * 2048 || d->ws_stride_e < nfr * nst * 128)) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
+    if (mx_out && extras) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: betas / out_alpha / acc_in are not supported together with an MX-quantised output");
     if (mx_out) {
       const int64_t n_out = swiglu ? d->N / 2 : d->N;
       if (n_out % 32) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: an MX-quantised output needs N_out %% 32 == 0 (got %lld)", (long long)n_out);
@@ -125,6 +136,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->w_layout == TK_W_TILED) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
     if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);
+    if (d->block_m >= 64 && extras) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: betas / out_alpha / acc_in need block_m 16 or 32 with tiled MXFP4 weights");
     if (d->block_m >= 64) {
       // the prefill kernels address activation rows with 32-bit byte offsets from x
       if (d->gather_indx && d->x_rows <= 0)

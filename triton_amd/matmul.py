@@ -16,8 +16,9 @@ Python validates, picks the tile (`opt_flags`), allocates the output with `torch
                                                 the narrow operand without a native partner is expanded to bf16 / fp16 by
                                                 the MX dequantiser kernel (activations per call, weights once, cached)
 
-Options of the reference signature that this build rejects with NotImplementedError: `c_acc_in`, `fused_comm`, `betas`, `out_alpha`, the NVFP4 output epilogue, flexpoint
-output / accumulator scales, split-k.  Batched 3-D activations run as a ragged problem with equal slices.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
+Options of the reference signature that this build rejects with NotImplementedError: `fused_comm`, the NVFP4 output epilogue, flexpoint
+output / accumulator scales, split-k.  `betas`, `out_alpha` and `c_acc_in` are applied in the reference's epilogue order by the kernels with the shared epilogue
+(tiled MXFP4 weights then run on the decode kernel's row blocks; `c_acc_in` must have the output's dtype).  Batched 3-D activations run as a ragged problem with equal slices.  Flexpoint input scales (`flex_ctx.lhs_data.scale`,
 `flex_ctx.rhs_data.scale`) are folded into the per-row / per-column scales of the epilogue.  MXFP8 / MXFP4 output epilogues run as the bf16 GEMM followed by the
 MX quantiser kernel on the same stream.
 """
@@ -283,7 +284,7 @@ def _k_contiguous(w: torch.Tensor) -> torch.Tensor:
 
 
 def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
-                   fused_activation, epilogue):
+                   fused_activation, epilogue, betas=None, out_alpha=None, c_acc_in=None):
     """`Epilogue(FnSpecs(QUANTIZE_MXFP8 | QUANTIZE_MXFP4, ...))` with `precision_config.c_mx_scale`
     (triton_kernels/matmul.py:53-56,364-369,500-505; kernel side matmul_details/_matmul.py:593-637): the output is
     quantised along N in blocks of 32, values in `out_dtype` (float8 or packed e2m1 in uint8) and one e8m0 scale
@@ -310,8 +311,8 @@ def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, pre
         scale_data = scale_out
     assert scale_data.dtype == torch.uint8, f"Unsupported output microscale dtype {scale_data.dtype}"
     plain = dataclasses.replace(precision_config, c_mx_scale=None, out_dtype=torch.bfloat16)
-    y = matmul(a, b, bias, a_ragged_metadata, None, gather_indx, scatter_indx, plain, None, gammas, None, None, None,
-               fused_activation, None, None)
+    y = matmul(a, b, bias, a_ragged_metadata, None, gather_indx, scatter_indx, plain, betas, gammas, out_alpha, None, None,
+               fused_activation, None, c_acc_in)
     n_out = y.shape[-1]
     if n_out % MXFP_BLOCK_SIZE != 0:
         raise NotImplementedError(f"MX-quantised output needs N_out % 32 == 0 (got {n_out})")
@@ -319,6 +320,7 @@ def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, pre
         f"c_mx_scale must be [{y.shape[0]}, {n_out // MXFP_BLOCK_SIZE}], got {tuple(scale_data.shape)}"
     vals, scales = downcast_to_mxfp(y, out_dtype, axis=-1)
     scale_data.view(scales.shape).copy_(scales)
+    # (the reference records these on the caller's PrecisionConfig as well: triton_kernels/matmul.py:364-369,764-765)
     precision_config.c_mx_scale = scale_out
     precision_config.c_microblock_size = MXFP_BLOCK_SIZE
     precision_config.c_value_pack_factor = 2 if fp4 else 1
@@ -466,14 +468,13 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if a_data.ndim == 3:
         return _matmul_batched(a_data, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, betas, gammas,
                                out_alpha, c, fused_comm, fused_activation, epilogue, c_acc_in)
-    if c_acc_in is not None:
-        raise NotImplementedError("c_acc_in is not supported")
     if fused_comm is not None:
         raise NotImplementedError("fused_comm is a multi-GPU feature and is not supported")
-    if betas is not None:
-        raise NotImplementedError("betas is not supported")
-    if out_alpha is not None:
-        raise NotImplementedError("out_alpha is not supported")
+    # betas / out_alpha / c_acc_in (triton_kernels/matmul.py:251-258; epilogue order matmul_details/_matmul.py:547-559,
+    # 581-591) are served by the kernels with the shared epilogue; see `extras` below
+    extras = betas is not None or out_alpha is not None or c_acc_in is not None
+    if c_acc_in is not None and scatter_indx is not None:
+        raise AssertionError("c_acc_in + scatter is not supported.")  # triton_kernels/matmul.py:531
     if precision_config is None:
         precision_config = PrecisionConfig()
     if fused_activation is None:
@@ -503,9 +504,11 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         mx_out_fused = (mx_act and epilogue.specs.name == FnName.QUANTIZE_MXFP8.name
                         and precision_config.out_dtype == torch.float8_e4m3fn and precision_config.c_mx_scale is not None
                         and precision_config.c_microblock_size in (None, MXFP_BLOCK_SIZE))
+        if mx_out_fused and extras:
+            raise NotImplementedError("betas / out_alpha / c_acc_in are not supported together with the fused MX-output epilogue")
         if not mx_out_fused:
             return _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, precision_config, gammas, c,
-                                  fused_activation, epilogue)
+                                  fused_activation, epilogue, betas, out_alpha, c_acc_in)
     elif epilogue.specs.fn is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
         raise NotImplementedError(f"epilogue {epilogue.specs.name!r} is not supported (MXFP8 / MXFP4 output quantisation only)")
     flex = precision_config.flex_ctx
@@ -592,6 +595,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
             raise NotImplementedError(f"MX-quantised output needs N_out % 32 == 0 (got {out_shape[1]})")
         assert c_scale.dtype == torch.uint8 and tuple(c_scale.shape[-2:]) == (y_rows, out_shape[1] // MXFP_BLOCK_SIZE) \
             and c_scale.stride(-1) == 1, f"c_mx_scale must be uint8 [{y_rows}, {out_shape[1] // MXFP_BLOCK_SIZE}]"
+        # (recorded on the caller's PrecisionConfig, as the reference does: triton_kernels/matmul.py:364-369)
         precision_config.c_microblock_size = MXFP_BLOCK_SIZE
         precision_config.c_value_pack_factor = 1
     caller_c = c is not None
@@ -719,6 +723,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         from .matmul_details.opt_flags import _get_opt_flags_constraints
         forced = _get_opt_flags_constraints().get("block_m")
         block_m = 256 if (forced == 256 or (forced is None and is_ragged and M <= 144 * n_slices)) else 128
+    elif tiled and extras:
+        block_m = min(block_m, 32)  # the decode kernel carries the shared epilogue; the prefill kernels do not take these options
     elif tiled:
         from .matmul_details.opt_flags import _get_opt_flags_constraints
         if block_m == 128 and _get_opt_flags_constraints().get("block_m") is None and is_ragged and M <= 144 * n_slices:
@@ -757,8 +763,25 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if c_scale is not None:
         d.y_mx_scale = c_scale.data_ptr()
         d.ys_stride_m = c_scale.stride(-2)
+    if betas is not None:
+        assert betas.shape[0] == M, f"betas must hold one value per row ({M}), got {tuple(betas.shape)}"
+        be = betas if betas.dtype in (torch.float32, torch.bfloat16) else betas.to(torch.float32)
+        be = be.contiguous()
+        d.betas = be.data_ptr()
+        d.betas_dtype = nt.TORCH_TO_TK[be.dtype]
+        keep.append(be)
+    if out_alpha is not None:
+        d.has_out_alpha = 1
+        d.out_alpha = float(out_alpha)
+    if c_acc_in is not None:
+        acc_in = c_acc_in.view(out_shape) if c_acc_in.ndim > 2 else c_acc_in
+        if tuple(acc_in.shape) != out_shape or acc_in.dtype != c.dtype or acc_in.stride(-1) != 1:
+            raise NotImplementedError(f"c_acc_in must have the output's shape {out_shape} and dtype {c.dtype} with unit stride along N")
+        d.acc_in = acc_in.data_ptr()
+        d.acc_in_stride_m = acc_in.stride(0)
+        keep.append(acc_in)
     combined = None
-    if (_combine_k and tiled and not mx_act and block_m <= 32 and act == nt.TK_ACT_NONE and scatter_indx is not None
+    if (_combine_k and not extras and tiled and not mx_act and block_m <= 32 and act == nt.TK_ACT_NONE and scatter_indx is not None
             and scatter_indx.shape[0] % _combine_k == 0
             and (scatter_indx.shape[0] // _combine_k) * ((N + 31) // 32) <= _COMBINE_COUNTER_WORDS):
         combined = torch.empty((scatter_indx.shape[0] // _combine_k, N), dtype=c.dtype, device=c.device)
