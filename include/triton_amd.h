@@ -319,7 +319,11 @@ typedef struct tk_gemm_desc {
    * [rows of y, N_out / 32].  NULL = plain bf16 output. */
   void* y_mx_scale;
   int64_t ys_stride_m;
-  /* Fused top-k combine behind the scatter (decode: tiled MXFP4 weights, block_m 16 or 32, no activation):
+  /* Fused top-k combine behind the scatter (bf16 activations, tiled MXFP4 weights, no activation).  At block_m >= 64
+   * the persistent kernel sums when all its workgroups have written their tiles (a device-wide arrival count in words
+   * 9..31 of tile_counters, which must be given; word 11 is raised, and stays, if a bounded wait for the other
+   * workgroups runs out; combine_counters is not used; N % 8 == 0, 16-byte aligned rows of combine_out, and the
+   * launch must not share the GPU with another launch that waits for its own workgroups).  At block_m 16 or 32:
    * scatter_indx maps expert-sorted row r to flat position t * combine_k + j; besides y [tokens * combine_k, N] the
    * kernel writes combine_out[t, :] = sum over j of y[t * combine_k + j, :] (fp32 sum in j order, bf16 result: what
    * tk_reduce_mid computes from y), by the wave that completes token t's rows last.  combine_counters:
@@ -351,7 +355,7 @@ typedef struct tk_gemm_desc {
   int64_t acc_in_stride_m;
 } tk_gemm_desc;
 
-#define TK_GEMM_TILE_COUNTER_WORDS 16
+#define TK_GEMM_TILE_COUNTER_WORDS 32
 
 /* Replaces the `_matmul[(grid,)](...)` launch of tk/matmul.py:659-726 (kernel tk/matmul_details/_matmul.py:43-672). */
 int32_t tk_moe_gemm(const tk_gemm_desc* desc, tk_stream_t stream);

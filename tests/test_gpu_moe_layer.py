@@ -568,3 +568,28 @@ def test_config3_full_shape_mxfp8_activations_sampled_tokens(api, device, gptoss
     # the second GEMM's 2880-term sums the difference is far below the bf16 GEMM tolerance used here)
     assert_close(ref, got, maxtol=3e-2, what="sampled token outputs, MXFP8 activations")
     assert_allclose_gate(ref, got, what="sampled token outputs, MXFP8 activations", max_bad_frac=LAYER_GATE_SLACK * 20)
+
+
+@pytest.mark.parametrize("T", [300, 4096])
+def test_fused_combine_at_prefill_equals_reduce(api, device, gptoss_weights, T):
+    """At prefill shapes `matmul_ogs(..., scatter_indx=...)` sums the k rows of every token at the end of the second
+    GEMM's own launch (the persistent grid waits until all its workgroups have written their tiles).  Bit-equal to
+    `reduce` over the scattered rows, three calls in a row on the same counters (left clean), error word clear."""
+    import triton_amd.matmul as mm
+    g = torch.Generator().manual_seed(6 + T)
+    E, k, d = 128, 4, 2880
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
+    logits = torch.randn((T, E), generator=g).to(device)
+    W = gptoss_weights["tiled"]
+    rdata, gather, scatter = api.routing(logits, k)
+    pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
+    h = api.matmul(x, W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, precision_config=pc1,
+                   fused_activation=api.act(1.702, 7.0))
+    y = api.matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=scatter.dst_indx, precision_config=pc2, gammas=rdata.gate_scal)
+    want, _ = api.reduce(y.view(T, k, -1), dim=1)
+    for rep in range(3):
+        got = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=pc2, gammas=rdata.gate_scal)
+        assert got.shape == (T, d)
+        assert torch.equal(got, want), f"call {rep}: fused combine differs from reduce"
+    ctr = mm._tile_counters(device).cpu()
+    assert int(ctr[9]) == 0 and int(ctr[10]) == 0 and int(ctr[11]) == 0, f"tile counters after the launches: {ctr.tolist()}"

@@ -52,7 +52,7 @@ struct GemmParams {
   int32_t w_nst;     // tile-native weight layout: K-stages of 128 per column fragment
   int32_t total_tiles;  // persistent kernels, non-ragged case: row blocks x column tiles
   int32_t idle_cus;     // persistent kernels: compute units to leave without a workgroup
-  int32_t* tile_counters;  // persistent kernels: 16 zeroed words for dynamic tile claiming (9 are used), or null
+  int32_t* tile_counters;  // persistent kernels: 32 zeroed words (tile claiming: 0..8; prefill combine: 9..31), or null
   uint32_t y_bytes;        // persistent MXFP4 kernels: bytes of the output buffer that rows may be written to (< 2 GiB)
   int32_t combine_k;          // decode kernel: > 0 = sum the k rows of every token into combine_out (fused top-k combine)
   uint16_t* combine_out;      // bf16 [tokens, N]

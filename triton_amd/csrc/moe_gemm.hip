@@ -73,10 +73,14 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.combine_stride = 0;
   p.combine_counters = nullptr;
   if (d->combine_k > 0) {
-    if (!(d->w_layout == TK_W_TILED && d->w_dtype == TK_E2M1 && (d->block_m == 16 || d->block_m == 32)))
-      return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine needs tiled MXFP4 weights and block_m 16 or 32");
-    if (!d->scatter_indx || !d->combine_out || !d->combine_counters || d->activation != TK_ACT_NONE)
-      return fail(TK_ERR_INVALID, "tk_moe_gemm: the fused top-k combine needs scatter_indx, combine_out and combine_counters, and no activation");
+    const bool decode_tile = d->block_m == 16 || d->block_m == 32;
+    if (!(d->w_layout == TK_W_TILED && d->w_dtype == TK_E2M1 && d->x_dtype == TK_BF16 && !d->x_mx_scale))
+      return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine needs bf16 activations and tiled MXFP4 weights");
+    // block_m 16 / 32: arrival counters per (token, fragment); block_m >= 64: the persistent kernel's tile counters
+    if (!d->scatter_indx || !d->combine_out || !(decode_tile ? d->combine_counters != nullptr : d->tile_counters != nullptr) || d->activation != TK_ACT_NONE)
+      return fail(TK_ERR_INVALID, "tk_moe_gemm: the fused top-k combine needs scatter_indx, combine_out, its counters (combine_counters at block_m 16 / 32, tile_counters above) and no activation");
+    if (!decode_tile && (d->N % 8 || d->combine_stride_m % 8 || (reinterpret_cast<uintptr_t>(d->combine_out) & 15)))
+      return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine at block_m >= 64 needs N %% 8 == 0 and 16-byte aligned rows of combine_out");
     if (d->scatter_len % d->combine_k) return fail(TK_ERR_INVALID, "tk_moe_gemm: scatter_len %d is not a multiple of combine_k %d", d->scatter_len, d->combine_k);
     const int64_t yb = (int64_t)d->scatter_len * d->y_stride_m * 2;
     if (yb >= (int64_t)1 << 31 || d->y_stride_m % 4 || (reinterpret_cast<uintptr_t>(d->y) & 7) || d->N % 4)

@@ -582,6 +582,84 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     }
   }
   if (dyn) claimer.finish();
+  // ---- top-k combine behind the scatter (reduce.py:1143-1165 after matmul_details/_matmul.py:535-569 in the reference,
+  // a launch of its own there): out[t, :] = sum over j of y[t * k + j, :], fp32 in j order, bf16 result.  The k rows of a
+  // token come from k experts, i.e. from tiles of workgroups all over the chip, so the sum runs when EVERY workgroup
+  // has written its tiles: the grid is persistent and fits the GPU (one workgroup per CU).
+  //   1. a workgroup whose stores have all reached its XCD's L2 counts itself in (per XCD and in total);
+  //   2. when all have, ONE workgroup per XCD (the first to claim it) has that L2 write its dirty lines back (a release
+  //      fence; one per L2, not one per wave: every fence walks the whole cache) and reports it;
+  //   3. when every XCD in use has reported, the rows of y are in memory: the workgroups sum the tokens blockIdx.x,
+  //      blockIdx.x + grid, ..., reading y around their own L2 (sc0 sc1: lines another XCD wrote are not coherent in it);
+  //   4. the last workgroup to leave clears the words for the next launch.
+  // Words of `tile_counters`: 9 arrivals, 10 departures, 11 error (raised, and kept, if a bounded wait runs out),
+  // 12 XCDs in use, 13 XCDs written back, 16..23 arrivals per XCD, 24..31 write-back claimed per XCD.
+  if constexpr (!SWIGLU) {
+    if (p.combine_k > 0 && p.tile_counters != nullptr) {
+      int32_t* ctr = p.tile_counters;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) {
+        int xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        xcc &= 7;
+        auto wait_for = [&](int32_t* word, int want) {
+          int spins = 0;
+          while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+            __builtin_amdgcn_s_sleep(16);
+            if (++spins > (1 << 22)) {
+              atomicOr(&ctr[11], 1);
+              break;
+            }
+          }
+        };
+        if (__hip_atomic_fetch_add(&ctr[16 + xcc], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+          __hip_atomic_fetch_add(&ctr[12], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(&ctr[9], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        wait_for(&ctr[9], grid);
+        if (__hip_atomic_fetch_add(&ctr[24 + xcc], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this XCD's L2 writes back its dirty lines
+          __hip_atomic_fetch_add(&ctr[13], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        wait_for(&ctr[13], __hip_atomic_load(&ctr[12], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      }
+      __syncthreads();
+      const int k = p.combine_k, T = p.scatter_len / k;
+      const int n8 = N >> 3;  // (N is a multiple of 8: host check)
+      const __amdgpu_buffer_rsrc_t ysrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
+      const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
+      constexpr int kAround = 1 | 16;  // sc0 | sc1
+      for (int t = blockIdx.x; t < T; t += grid) {
+        for (int c = tid; c < n8; c += NT) {
+          float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          for (int j0 = 0; j0 < k; j0 += 4) {
+            u32x4_t v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t off = j0 + q < k ? (uint32_t)(t * k + j0 + q) * row_bytes + (uint32_t)c * 16u : kDroppedStore;
+              v[q] = __builtin_amdgcn_raw_buffer_load_b128(ysrc, off, 0, kAround);  // (dropped offsets read zero)
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                sum[2 * e] += bits_f32(v[q][e] << 16);
+                sum[2 * e + 1] += bits_f32(v[q][e] & 0xFFFF0000u);
+              }
+          }
+          *reinterpret_cast<u32x4_t*>(p.combine_out + (int64_t)t * p.combine_stride + c * 8) =
+              u32x4_t{pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]), pack_bf16x2(sum[4], sum[5]), pack_bf16x2(sum[6], sum[7])};
+        }
+      }
+      __syncthreads();
+      if (tid == 0) {
+        if (__hip_atomic_fetch_add(&ctr[10], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == grid - 1) {
+          for (int w = 9; w < 32; ++w)
+            if (w != 11) __hip_atomic_store(&ctr[w], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
+  }
 }
 
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD>

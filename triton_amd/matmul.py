@@ -121,7 +121,7 @@ def _tile_counters(device: torch.device) -> torch.Tensor:
     key = (device.index, nt.stream_ptr(device))
     buf = _TILE_COUNTERS.get(key)
     if buf is None:
-        buf = torch.zeros(16, dtype=torch.int32, device=device)
+        buf = torch.zeros(32, dtype=torch.int32, device=device)
         _TILE_COUNTERS[key] = buf
     return buf
 
@@ -780,17 +780,24 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         d.acc_in = acc_in.data_ptr()
         d.acc_in_stride_m = acc_in.stride(0)
         keep.append(acc_in)
+    if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES and not mx_act:
+        d.tile_counters = _tile_counters(a.device).data_ptr()
     combined = None
-    if (_combine_k and not extras and tiled and not mx_act and block_m <= 32 and act == nt.TK_ACT_NONE and scatter_indx is not None
-            and scatter_indx.shape[0] % _combine_k == 0
-            and (scatter_indx.shape[0] // _combine_k) * ((N + 31) // 32) <= _COMBINE_COUNTER_WORDS):
+    can_combine = (_combine_k and not extras and tiled and not mx_act and act == nt.TK_ACT_NONE and scatter_indx is not None
+                   and scatter_indx.shape[0] % _combine_k == 0 and a.dtype == torch.bfloat16)
+    if can_combine and block_m <= 32:
+        # decode kernel: the wave that completes a token's rows last sums them (arrival counters per token and fragment)
+        can_combine = (scatter_indx.shape[0] // _combine_k) * ((N + 31) // 32) <= _COMBINE_COUNTER_WORDS
+    elif can_combine:
+        # prefill kernel: the persistent grid sums when all its workgroups have written their tiles
+        can_combine = bool(d.tile_counters) and N % 8 == 0 and y_buf is c
+    if can_combine:
         combined = torch.empty((scatter_indx.shape[0] // _combine_k, N), dtype=c.dtype, device=c.device)
         d.combine_k = int(_combine_k)
         d.combine_out = combined.data_ptr()
         d.combine_stride_m = combined.stride(0)
-        d.combine_counters = _combine_counters(a.device).data_ptr()
-    if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES and not mx_act:
-        d.tile_counters = _tile_counters(a.device).data_ptr()
+        if block_m <= 32:
+            d.combine_counters = _combine_counters(a.device).data_ptr()
     with nt.on_device(a.device):
         nt.check(nt.lib().tk_moe_gemm(d, nt.stream_ptr(a.device)))
     del keep
