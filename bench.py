@@ -192,6 +192,23 @@ def time_steps(fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_graph_steps(fn, steps, warmup):
+    """`fn()` (returns a tensor) captured twice in HIP graphs; a step is one replay, the two captures in turn (a graph
+    cannot overlap with its own previous launch, so replays of ONE graph would charge an idle gap to every step).
+    Every capture's replay is compared with the eager result first.  Returns (ms per replayed step, ms per eager step)."""
+    eager = fn().clone()
+    graphs = [capture(fn) for _ in range(2)]
+    for _ in range(2):  # replays with eager work in between
+        for graph, out in graphs:
+            graph.replay()
+            torch.cuda.synchronize()
+            if not torch.equal(out, eager):
+                raise RuntimeError("graph replay differs from the eager result")
+        fn()
+    ms = time_steps(lambda i=[0]: (graphs[i[0] % 2][0].replay(), i.__setitem__(0, i[0] + 1)), steps, warmup)
+    return ms, time_steps(fn, steps, warmup)
+
+
 def cpu_baseline(seed=2, min_seconds=10.0):
     """CPU oracle on a bounded sample of config 3: 32 of the 128 experts and 1024 tokens (top-4), which keeps
     the ~128 routed rows per expert of the full workload; passes are repeated until `min_seconds` of CPU work."""
@@ -377,10 +394,11 @@ def bench_fp8(device, steps, warmup):
                    precision_config=PrecisionConfig(a_mx_tensor_scale=sh, b_mx_tensor_scale=s2, out_dtype=torch.bfloat16))
         return reduce(y.view(T, k, -1), dim=1)[0]
 
-    ms = time_steps(step, steps, warmup)
+    ms, ms_eager = time_graph_steps(step, steps, warmup)
     board = board_state_under(step)
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
-    return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8",
+    return dict(ms_per_step=round(ms, 4), ms_per_step_eager=round(ms_eager, 4), step_mode="hip_graph_replay",
+                TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8",
                 frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), board_under_step=board,
                 mfma_sustained_probe=mfma_sustained_probe(device, kind=1))
 
@@ -390,11 +408,10 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
     K) and multiplied with the MXFP4 weights by v_mfma_scale_f32_32x32x64_f8f6f4, both operands in their storage
     formats; the first GEMM's epilogue quantises its fp32 accumulator to MXFP8 for the second.  Not the headline:
     config 3 states bf16 activations, and this path is checked against an oracle fed the same quantised activations.
-    One step = router, quantise x, GEMM1 (+bias, swiglu, MX output), GEMM2 (+bias, gate weight), combine."""
-    from triton_kernels.legacy import routing
+    One step = router, quantise x, GEMM1 (+bias, swiglu, MX output), GEMM2 (+bias, gate weight, top-k combine)."""
+    from triton_kernels.legacy import matmul_ogs, routing
     from triton_kernels.matmul import Epilogue, FnName, FnSpecs, FusedActivation, PrecisionConfig, matmul
     from triton_kernels.numerics_details.mxfp import downcast_to_mxfp, quantize_mxfp8_fn
-    from triton_kernels.reduce import reduce
     from triton_kernels.swiglu import swiglu_fn
     T, d = x.shape
     W = weights
@@ -408,11 +425,11 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
         xq, xs = downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
         h = matmul(xq, W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, fused_activation=act, epilogue=epi,
                    precision_config=PrecisionConfig(a_mx_scale=xs, b_mx_scale=W["w1s"], c_mx_scale=h_scale, out_dtype=torch.float8_e4m3fn))
-        y = matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=scatter.dst_indx, gammas=rdata.gate_scal,
-                   precision_config=PrecisionConfig(a_mx_scale=h_scale, b_mx_scale=W["w2s"], out_dtype=torch.bfloat16))
-        return reduce(y.view(T, k, -1), dim=1)[0]
+        # (the legacy entry point sums the k rows of a token at the end of the scatter-GEMM's launch, as in the headline step)
+        return matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, gammas=rdata.gate_scal,
+                          precision_config=PrecisionConfig(a_mx_scale=h_scale, b_mx_scale=W["w2s"], out_dtype=torch.bfloat16))
 
-    ms = time_steps(step, steps, warmup)
+    ms, ms_eager = time_graph_steps(step, steps, warmup)
     board = board_state_under(step)
     flops = 2.0 * T * k * (d * f2 + (f2 // 2) * d)
     # algorithmic bytes with one-byte activations: x_q + scales, W1, h_q twice, W2, y twice, out
@@ -420,7 +437,8 @@ def bench_scaled_mfma(device, weights, x, logits, k, steps, warmup):
     E = W["b1"].shape[0]
     nbytes = (R * d * 33 / 32 + E * (d * f2 * 17 / 32 + f2 * 2) + 2 * R * (f2 // 2) * 33 / 32 + E * ((f2 // 2) * d * 17 / 32 + d * 2) + 2 * R * d * 2 + T * d * 2)
     t_roof_ms = max(flops / 5.0e15, nbytes / (PEAK_HBM_GBPS * 1e9)) * 1e3
-    return dict(ms_per_step=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1), mfma_class="fp8 (MXFP8 x MXFP4, scaled MFMA)",
+    return dict(ms_per_step=round(ms, 4), ms_per_step_eager=round(ms_eager, 4), step_mode="hip_graph_replay", TFLOPs=round(flops / ms / 1e9, 1),
+                mfma_class="fp8 (MXFP8 x MXFP4, scaled MFMA)",
                 frac_mfma_fp8=round(flops / ms / 1e9 / 5000.0, 4), t_roof_ms=round(t_roof_ms, 4), frac=round(t_roof_ms / ms, 4),
                 bound="hbm" if nbytes / (PEAK_HBM_GBPS * 1e9) > flops / 5.0e15 else "mfma", board_under_step=board)
 

@@ -593,3 +593,30 @@ def test_fused_combine_at_prefill_equals_reduce(api, device, gptoss_weights, T):
         assert torch.equal(got, want), f"call {rep}: fused combine differs from reduce"
     ctr = mm._tile_counters(device).cpu()
     assert int(ctr[9]) == 0 and int(ctr[10]) == 0 and int(ctr[11]) == 0, f"tile counters after the launches: {ctr.tolist()}"
+
+
+@pytest.mark.parametrize("T", [300, 4096])
+def test_matmul_ogs_with_mxfp8_activations_equals_matmul_then_reduce(api, device, gptoss_weights, T):
+    """The scaled-MFMA path through the legacy entry point: hidden activations MX-quantised to e4m3 by the first GEMM's
+    epilogue, second GEMM (MXFP8 x tiled MXFP4) with scatter, gate weight and the sum over a token's k rows, bit-equal to
+    `matmul` followed by `reduce`, three calls in a row."""
+    from triton_amd.matmul import Epilogue, FnName, FnSpecs
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp, quantize_mxfp8_fn
+    g = torch.Generator().manual_seed(16 + T)
+    E, k, d, f2 = 128, 4, 2880, 5760
+    x = torch.randn((T, d), generator=g).to(torch.bfloat16).to(device)
+    logits = torch.randn((T, E), generator=g).to(device)
+    W = gptoss_weights["tiled"]
+    rdata, gather, scatter = api.routing(logits, k)
+    xq, xs = downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
+    epi = Epilogue(FnSpecs(FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn, (), ()), tuple(), tuple(), effective_itemsize=1.0)
+    h_scale = torch.empty((T * k, (f2 // 2) // 32), dtype=torch.uint8, device=device)
+    h = api.matmul(xq, W["w1"], W["b1"], rdata.expt_data, gather_indx=rdata.token_indx, fused_activation=api.act(1.702, 7.0), epilogue=epi,
+                   precision_config=api.PrecisionConfig(a_mx_scale=xs, b_mx_scale=W["w1s"], c_mx_scale=h_scale, out_dtype=torch.float8_e4m3fn))
+    pc2 = api.PrecisionConfig(a_mx_scale=h_scale, b_mx_scale=W["w2s"], out_dtype=torch.bfloat16)
+    y = api.matmul(h, W["w2"], W["b2"], rdata.expt_data, scatter_indx=scatter.dst_indx, precision_config=pc2, gammas=rdata.gate_scal)
+    want, _ = api.reduce(y.view(T, k, -1), dim=1)
+    for rep in range(3):
+        got = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=pc2, gammas=rdata.gate_scal)
+        assert got.shape == (T, d)
+        assert torch.equal(got, want), f"call {rep}: matmul_ogs differs from matmul + reduce"

@@ -135,6 +135,23 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     }
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
+    {
+      // The persistent form of the kernel (units of work two ahead, branch-free epilogue through buffer resources) needs
+      // 32-bit addressable activations and scales, aligned output rows in less than 2 GiB, the ragged metadata in LDS and
+      // the plain epilogue; anything else runs the tile-at-a-time form.
+      const int64_t x_rows = d->x_rows > 0 ? d->x_rows : (d->gather_indx ? 0 : d->M);
+      const int64_t n_out = swiglu ? d->N / 2 : d->N;
+      const int64_t y_rows = d->scatter_indx ? d->scatter_len : d->M;
+      const int64_t elem = mx_out ? 1 : 2, piece = swiglu ? 4 : 8;
+      const int64_t y_bytes = y_rows * d->y_stride_m * elem;
+      bool fast = x_rows > 0 && x_rows * d->x_stride_m < ((int64_t)1 << 32) && x_rows * d->xs_stride_m < ((int64_t)1 << 32) && d->x_stride_m >= 0 &&
+                  d->xs_stride_m >= 0 && !extras && d->n_slices <= kMetaSlices && y_bytes > 0 && y_bytes < ((int64_t)1 << 31) && d->y_stride_m >= 0;
+      if (mx_out)
+        fast = fast && p.y_vec && y_rows * d->ys_stride_m < ((int64_t)1 << 31) && d->ys_stride_m >= 0;
+      else
+        fast = fast && p.y_vec && d->y_stride_m >= cdiv(n_out, piece) * piece;
+      p.y_bytes = fast ? (uint32_t)y_bytes : 0u;
+    }
     return gemm_launch_mx8n(p, d->block_m, d->grid_m, swiglu, mx_out, st);
   }
   if (d->w_layout == TK_W_TILED) {

@@ -278,7 +278,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8n_kernel(const GemmParams p) 
     const int sh = xsshift[slot] < 4 ? xsshift[slot] : 4;
     const uint64_t wide = ((uint64_t)0x7F7F7F7Fu << 32) | xsreg[slot];
     const uint32_t v = (uint32_t)(wide >> (8 * sh));
-    if (tid < BM) *reinterpret_cast<uint32_t*>(lds + buf * XBYTES + tid * XPITCH + KC) = v;
+    // (no branch inside the K loop: threads past the tile's rows write into the unused pad bytes of a row)
+    const int at = tid < BM ? tid * XPITCH + KC : (tid - BM) * XPITCH + KC + 4;
+    *reinterpret_cast<uint32_t*>(lds + buf * XBYTES + at) = v;
   };
   auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
     constexpr int SL = decltype(slot_c)::value;
@@ -427,6 +429,547 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8n_kernel(const GemmParams p) 
   }  // rounds
 }
 
+// MX-quantised output of the persistent kernel below: `mx_out_epilogue` with the operands of rows and columns taken
+// from LDS (bias_s by tile column, gam_s / dst_s by tile row, fetched a unit ahead) and with no branch around a store:
+// rows without a destination, columns past the end and the lanes that do not write a block's scale byte store to an
+// offset beyond the range of their buffer resource, which the hardware drops.
+template <int MFW, int NFW, bool SWIGLU>
+__device__ __forceinline__ void staged_mx_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc,
+                                                   __amdgpu_buffer_rsrc_t ysrsrc, const float* bias_s, const float* gam_s, const int* dst_s,
+                                                   int ncol_tile, int ncol0, int lr, int h) {
+  const int NOUT = SWIGLU ? p.N / 2 : p.N;
+  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
+  const float limit = p.has_limit ? p.limit : INFINITY;
+  constexpr int VO = SWIGLU ? 4 : 8;
+  constexpr int NB = SWIGLU ? 1 : NFW;
+  // every LDS operand up front: one round trip for the unit
+  f32x4_t bh[NFW][2][2];
+  float gh[MFW];
+  int dh[MFW];
+#pragma unroll
+  for (int f = 0; f < NFW; ++f)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      bh[f][u][0] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 4 * h);
+      bh[f][u][1] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 8 + 4 * h);
+    }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    gh[j] = gam_s[j * 32 + lr];
+    dh[j] = dst_s[j * 32 + lr];
+  }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const float g = gh[j];
+    const int dst = dh[j];
+    float o[NFW][2][VO];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(acc[f][j][8 * u + i] + bh[f][u][0][i]), f32_bits(acc[f][j][8 * u + 4 + i] + bh[f][u][1][i]), false, false);
+          v[i] = bits_f32(sw[0]);
+          v[4 + i] = bits_f32(sw[1]);
+        }
+#pragma unroll
+        for (int i = 0; i < VO; ++i) o[f][u][i] = SWIGLU ? swiglu_f(v[2 * i], v[2 * i + 1], nalpha_log2e, limit) * g : v[i] * g;
+      }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      // block maximum of |o|: fmaxf returns its other operand for a NaN, so a NaN never wins and the block's scale comes
+      // from its finite values.  (N_out is a multiple of 32: a block lies below it whole or not at all, and one that does
+      // not is not stored.)
+      float m = 0.f;
+#pragma unroll
+      for (int f = 0; f < NFW; ++f) {
+        if (!SWIGLU && f != b) continue;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < VO; ++i) m = __builtin_fmaxf(m, __builtin_fabsf(o[f][u][i]));
+      }
+      {
+        // the other lane half's maximum: after the swap the first register holds both halves' lanes 0..31, the second both
+        // halves' lanes 32..63
+        auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(m), f32_bits(m), false, false);
+        m = __builtin_fmaxf(bits_f32(sw[0]), bits_f32(sw[1]));
+      }
+      const uint32_t sbits = mx_scale_bits(m, TK_E4M3, TK_MX_ROUND_UP);
+      const float inv = mx_inv_scale(sbits);
+      const int blk_col0 = SWIGLU ? ncol0 / 2 : ncol0 + b * 32;
+      const uint32_t soff = (dst >= 0 && h == 0 && blk_col0 < NOUT) ? (uint32_t)dst * (uint32_t)p.ys_stride_m + (uint32_t)(blk_col0 >> 5) : kDroppedStore;
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(sbits >> 23), ysrsrc, soff, 0, 0);
+#pragma unroll
+      for (int f = 0; f < NFW; ++f) {
+        if (!SWIGLU && f != b) continue;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int col0 = SWIGLU ? (ncol0 + f * 32 + 16 * u + 8 * h) / 2 : ncol0 + f * 32 + 16 * u + 8 * h;
+          // No clamp to +-448 in front of the conversion: the scale is the smallest power of two >= max / 448 (the rounded
+          // quotient of an fp32 by 448 = 1.75 * 2^8 is a power of two only when the exact one is), scaling by a power of
+          // two is exact, so |o * inv| <= 448 for every finite block; with an infinite maximum inv is 0.
+          float qv[VO];
+#pragma unroll
+          for (int i = 0; i < VO; ++i) qv[i] = o[f][u][i] * inv;
+          const uint32_t off = (dst >= 0 && col0 < NOUT) ? (uint32_t)dst * (uint32_t)p.y_stride_m + (uint32_t)col0 : kDroppedStore;
+          int w0 = 0;
+          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[0], qv[1], w0, false);
+          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[2], qv[3], w0, true);
+          if constexpr (VO == 8) {
+            int w1 = 0;
+            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[4], qv[5], w1, false);
+            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[6], qv[7], w1, true);
+            __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{(uint32_t)w0, (uint32_t)w1}, yrsrc, off, 0, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b32((uint32_t)w0, yrsrc, off, 0, 0);
+          }
+        }
+      }
+    }
+  }
+}
+
+#ifdef TK_MX8_STAMPS
+// diagnostic build only: per workgroup, sums of shader-clock cycles spent in [0] the K loops' prologues, [1] the K
+// loops, [2] the preparation of the next unit, [3] the epilogues; [4] units, [5] K-stages, [6] whole kernel
+__device__ long long mx8_stamps[1024][8];
+#define MX8_T() ((long long)__builtin_amdgcn_s_memtime())
+#define MX8_ADD(n, v) do { if (threadIdx.x == 0) mx8_stamps[blockIdx.x][n] += (v); } while (0)
+#else
+#define MX8_T() 0ll
+#define MX8_ADD(n, v) do {} while (0)
+#endif
+
+// The same K loop inside persistent workgroups that run their units of work two ahead, as the bf16-activation kernel
+// does: ragged metadata in LDS, a unit's gather indices fetched two units ahead and its epilogue operands one unit ahead,
+// its first K-stage issued before the previous unit's epilogue, tiles claimed from per-XCD queues when they do not
+// divide evenly, and an epilogue without branches around stores.  Needs what that scheme needs from the host: at most
+// kMetaSlices slices, activations (and their scales) addressable with 32-bit byte offsets, aligned output rows in a
+// buffer of less than 2 GiB, no betas / out_alpha / acc_in.
+template <int BLKM, int MFW, int NFW, bool SWIGLU, bool MXOUT>
+__global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) {
+  typedef Frag<32> FR;
+  constexpr int FM = 32, NT = 256, BM = MFW * 32, BN = 128 * NFW, KC = 128, NS = 2;
+  constexpr int XPITCH = KC + 16;
+  constexpr int XBYTES = BM * XPITCH;
+  constexpr int XCH = BM / 32;
+  // Register rings: weights WD stages deep (stage c uses slot c % WD, loads run WD - 1 stages ahead), activations XD
+  // stages deep on their way to LDS.  The stage body is unrolled UNR = lcm(WD, XD, 2) times so that every index is static.
+  constexpr int WD = 4, XD = 2, UNR = 4;  // (6 / 3 / 6 fits the registers too and measured 2 % faster on the first GEMM, 3 % slower on the second)
+  static_assert(UNR % WD == 0 && UNR % XD == 0 && UNR % 2 == 0, "ring depths divide the unroll factor");
+  static_assert(BM <= NT && BN <= NT, "one thread per tile row and per tile column fetches the epilogue operands");
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int32_t soffs_s[kMetaSlices], ssize_s[kMetaSlices], boffs_s[kMetaSlices + 1];
+  __shared__ __attribute__((aligned(16))) float bias_s[2][BN];
+  __shared__ float gam_s[2][BM];
+  __shared__ int32_t dst_s[2][BM], gidx_s[2][BM];
+  __shared__ int next_tile_s[2];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int nw = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 31, h = lane >> 5;
+  const int K = p.K, N = p.N;
+  const int nst = p.w_nst;
+  const int nfr = (N + 31) >> 5;
+  const int xc = tid & 7;
+  const int xlds0 = (tid >> 3) * XPITCH + xc * 16;  // activation piece j at xlds0 + j*32*XPITCH
+  const int kblocks = (K + 31) >> 5;
+  const int grid = (int)gridDim.x;
+  const bool ragged = p.slice_sizes != nullptr;
+  const int nblk = ragged ? p.block_offs[p.n_slices] : 0;
+  const int live = ragged ? nblk * p.grid_n : p.total_tiles;
+  if (ragged) {
+    for (int i = tid; i < p.n_slices; i += NT) {
+      soffs_s[i] = p.slice_offs[i];
+      ssize_s[i] = p.slice_sizes[i];
+      boffs_s[i] = p.block_offs[i];
+    }
+    if (tid == 0) boffs_s[p.n_slices] = nblk;
+  }
+  const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ysrsrc = __builtin_amdgcn_make_buffer_rsrc(p.y_mx_scale, 0, MXOUT ? 0x7FFFFFFF : 0, 0x00020000);
+
+  struct Unit {
+    int expert, blk_off, blk_rows, pid_n, start_m, pass_off;
+    bool valid;
+  };
+  auto tile_unit = [&](int pid) __attribute__((always_inline)) -> Unit {
+    Unit u;
+    int eM;
+    if (ragged) {
+      // tiles are ordered (expert, column tile, row block); the expert is the last slice whose first block is not past
+      // block pid / grid_n: a binary search in the block offsets kept in LDS
+      const int blk = pid / p.grid_n;
+      int lo = 0, hi = p.n_slices;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (boffs_s[mid] <= blk) lo = mid; else hi = mid;
+      }
+      u.expert = lo;
+      const int first = boffs_s[lo];
+      const int nb = boffs_s[lo + 1] - first;
+      const int local = pid - first * p.grid_n;
+      u.pid_n = local / nb;
+      u.blk_off = (local - u.pid_n * nb) * BLKM;
+      u.start_m = soffs_s[lo];
+      eM = ssize_s[lo];
+    } else {
+      u.pid_n = pid % p.grid_n;
+      u.expert = 0;
+      u.blk_off = (pid / p.grid_n) * BLKM;
+      u.start_m = 0;
+      eM = p.M;
+    }
+    u.blk_rows = (eM - u.blk_off) < BLKM ? (eM - u.blk_off) : BLKM;
+    u.pass_off = 0;
+    u.valid = true;
+    u.expert = __builtin_amdgcn_readfirstlane(u.expert);
+    u.blk_off = __builtin_amdgcn_readfirstlane(u.blk_off);
+    u.blk_rows = __builtin_amdgcn_readfirstlane(u.blk_rows);
+    u.pid_n = __builtin_amdgcn_readfirstlane(u.pid_n);
+    u.start_m = __builtin_amdgcn_readfirstlane(u.start_m);
+    return u;
+  };
+  auto advance = [&](const Unit& u, int pid_after) __attribute__((always_inline)) -> Unit {
+    Unit n = u;
+    if (u.pass_off + BM < u.blk_rows) {
+      n.pass_off = u.pass_off + BM;
+    } else if (pid_after >= 0) {
+      n = tile_unit(pid_after);
+    } else {
+      n.valid = false;
+    }
+    return n;
+  };
+
+  // (tiles are dealt statically here: claimed tiles start at different times and drift apart in K, and the workgroups of
+  // an XCD then no longer meet each other's activation rows in its L2; measured 3 % slower at the gpt-oss shape)
+  constexpr bool dyn = false;
+  TileClaimer claimer;
+  int round0 = 0;
+  int pid, pid_next;
+  if (dyn) {
+    pid = claimer.init(p.tile_counters, live);
+    pid_next = pid >= 0 ? claimer.second() : -1;
+  } else {
+    const int in0 = live < grid ? live : grid;
+    pid = (int)blockIdx.x < in0 ? xcd_remap(blockIdx.x, in0) : -1;
+    round0 = grid;
+    const int in1 = live - round0 < grid ? live - round0 : grid;
+    pid_next = (pid >= 0 && (int)blockIdx.x < in1) ? round0 + xcd_remap(blockIdx.x, in1) : -1;
+  }
+  int n_tile = 0;
+  if (ragged) __syncthreads();
+
+  // per-unit operand addresses: uniform 64-bit bases plus 32-bit byte offsets per lane
+  uint32_t xoff[XCH];   // this thread's row of piece j in x (one byte per element)
+  uint32_t xsoff = 0;   // row `tid` in the activation scales
+  const uint8_t* wbase[NFW];
+  const uint8_t* sbase[NFW];
+  const uint32_t lane16 = lane * 16, lr4 = lr * 4;
+  auto unit_gather_index = [&](const Unit& u) __attribute__((always_inline)) -> int {
+    int row = u.blk_off + u.pass_off + tid;
+    row = row < u.blk_off + u.blk_rows ? row : u.blk_off + u.blk_rows - 1;
+    const int srow = u.start_m + row;
+    return p.gather ? p.gather[srow] : srow;
+  };
+  auto unit_pointers = [&](const Unit& u, int set) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < XCH; ++j) xoff[j] = (uint32_t)gidx_s[set][(tid >> 3) + 32 * j] * (uint32_t)p.x_stride_m;
+    xsoff = (uint32_t)gidx_s[set][tid < BM ? tid : BM - 1] * (uint32_t)p.xs_stride_m;
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) {
+      int F = u.pid_n * (BN / 32) + nw * NFW + f;
+      F = F < nfr ? F : nfr - 1;
+      wbase[f] = p.w + (int64_t)u.expert * p.w_stride_e + (int64_t)F * nst * 2048;
+      sbase[f] = p.w_scale + (int64_t)u.expert * p.ws_stride_e + (int64_t)F * nst * 128;
+    }
+  };
+  uint32_t bias_raw = 0, gam_raw = 0;
+  int dst_raw = 0, gidx_v = 0;
+  auto unit_operands = [&](const Unit& u) __attribute__((always_inline)) {
+    const int off_m = u.blk_off + u.pass_off, blk_end = u.blk_off + u.blk_rows;
+    if (p.bias) {
+      int n = u.pid_n * BN + (tid < BN ? tid : BN - 1);
+      n = n < N ? n : N - 1;
+      const int64_t i = (int64_t)u.expert * p.bias_stride_e + n;
+      bias_raw = p.bias_is_f32 ? static_cast<const uint32_t*>(p.bias)[i] : (uint32_t)static_cast<const uint16_t*>(p.bias)[i];
+    }
+    int row = off_m + (tid < BM ? tid : BM - 1);
+    row = row < blk_end ? row : blk_end - 1;
+    const int srow = u.start_m + row;
+    if (p.gammas) gam_raw = p.gammas_is_f32 ? static_cast<const uint32_t*>(p.gammas)[srow] : (uint32_t)static_cast<const uint16_t*>(p.gammas)[srow];
+    if (p.scatter) dst_raw = p.scatter[srow < p.scatter_len ? srow : p.scatter_len - 1];
+  };
+  auto stage_operands = [&](const Unit& u, int set) __attribute__((always_inline)) {
+    int t = tid;
+    asm volatile("" : "+v"(t));
+    if (t < BN) bias_s[set][t] = p.bias ? bits_f32(p.bias_is_f32 ? bias_raw : bias_raw << 16) : 0.f;
+    if (t < BM) {
+      const int off_m = u.blk_off + u.pass_off, blk_end = u.blk_off + u.blk_rows;
+      const bool ok = off_m + t < blk_end;
+      const int srow = u.start_m + off_m + t;
+      int dst = srow;
+      if (p.scatter) dst = srow < p.scatter_len ? dst_raw : -1;
+      gam_s[set][t] = p.gammas ? bits_f32(p.gammas_is_f32 ? gam_raw : gam_raw << 16) : 1.0f;
+      dst_s[set][t] = ok ? dst : -1;
+      gidx_s[set][t] = gidx_v;
+    }
+  };
+
+  typename FR::acc_t acc[NFW][MFW];
+  u32x4_t xreg[XD][XCH];
+  uint32_t xsreg[XD] = {};
+  int xsshift[XD] = {};
+  u32x4_t wraw[WD][NFW][NS];
+  uint32_t sd[WD][NFW];
+  i32x8_t xf[2][MFW];
+  uint32_t xs[2][MFW];
+
+  auto load_x_piece = [&](int j, int s, int slot) __attribute__((always_inline)) {
+    int k0 = s * KC + xc * 16;
+    k0 = k0 < K - 16 ? k0 : K - 16;
+    xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(p.x + (xoff[j] + (uint32_t)k0));
+  };
+  auto load_x_scale = [&](int s, int slot) __attribute__((always_inline)) {
+    int b0 = s * 4;
+    b0 = b0 < kblocks - 4 ? b0 : kblocks - 4;
+    uint32_t v;
+    __builtin_memcpy(&v, p.x_mx_scale + (xsoff + (uint32_t)b0), 4);
+    xsreg[slot] = v;
+    xsshift[slot] = s * 4 - b0;
+  };
+  auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 32 * XPITCH) = xreg[slot][j];
+  };
+  auto store_x_scale = [&](int buf, int slot) __attribute__((always_inline)) {
+    const int sh = xsshift[slot] < 4 ? xsshift[slot] : 4;
+    const uint64_t wide = ((uint64_t)0x7F7F7F7Fu << 32) | xsreg[slot];
+    const uint32_t v = (uint32_t)(wide >> (8 * sh));
+    // (no branch inside the K loop: threads past the tile's rows write into the unused pad bytes of a row)
+    const int at = tid < BM ? tid * XPITCH + KC : (tid - BM) * XPITCH + KC + 4;
+    *reinterpret_cast<uint32_t*>(lds + buf * XBYTES + at) = v;
+  };
+  auto load_w = [&](auto slot_c, int s) __attribute__((always_inline)) {
+    constexpr int SL = decltype(slot_c)::value;
+    s = s < nst ? s : nst - 1;
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) {
+      wraw[SL][f][0] = *reinterpret_cast<const u32x4_t*>(wbase[f] + (int64_t)s * 2048 + lane16);
+      wraw[SL][f][1] = *reinterpret_cast<const u32x4_t*>(wbase[f] + (int64_t)s * 2048 + 1024 + lane16);
+      sd[SL][f] = *reinterpret_cast<const uint32_t*>(sbase[f] + (int64_t)s * 128 + lr4);
+    }
+  };
+  auto read_xf = [&](int buf, int q, int j, i32x8_t (&out)[MFW]) __attribute__((always_inline)) {
+    const uint8_t* a = lds + buf * XBYTES + (j * FM + lr) * XPITCH + q * 32 + h * 16;
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(a);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(a + 64);
+    out[j] = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto read_xs = [&](int buf, int j, uint32_t (&out)[MFW]) __attribute__((always_inline)) {
+    out[j] = *reinterpret_cast<const uint32_t*>(lds + buf * XBYTES + (j * FM + lr) * XPITCH + KC) >> (16 * h);
+  };
+
+  template_int<0> S0;
+  template_int<1> S1;
+  template_int<2> S2;
+  template_int<3> S3;
+
+  auto stage = [&](auto nj_c, auto ws_c, int c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    constexpr int WSU = decltype(ws_c)::value;  // c % UNR
+    constexpr int WS4 = WSU % WD;               // weight ring slot of this stage
+    constexpr int PAR = WSU & 1;                // LDS buffer and activation scale set
+    using WSL = template_int<(WSU + WD - 1) % WD>;
+    constexpr int XS = (WSU + 1) % XD;
+    constexpr int NM = NJ * NFW;
+    constexpr int NOPS = 2 * NJ + 2;
+    uint32_t sdh[NFW];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f) sdh[f] = sd[WS4][f] >> (16 * h);
+    static_for<0, NS>([&](auto q_c) __attribute__((always_inline)) {
+      constexpr int q = decltype(q_c)::value;
+      constexpr int cur = q & 1, nxt = cur ^ 1;
+      auto op = [&](auto o_c) __attribute__((always_inline)) {
+        constexpr int o = decltype(o_c)::value;
+        if constexpr (o < NJ) {
+          if constexpr (q == 0) {
+            read_xf(PAR, 1, o, xf[nxt]);
+          } else {
+            read_xf(PAR ^ 1, 0, o, xf[nxt]);
+            read_xs(PAR ^ 1, o, xs[PAR ^ 1]);
+          }
+        } else if constexpr (o < 2 * NJ) {
+          if constexpr (q == 0) {
+            constexpr int j = o - NJ;
+            store_x_piece(j, PAR ^ 1, XS);
+            load_x_piece(j, c + 1 + XD, XS);
+          }
+        } else if constexpr (o == 2 * NJ) {
+          if constexpr (q == 0) {
+            store_x_scale(PAR ^ 1, XS);
+            load_x_scale(c + 1 + XD, XS);
+          }
+        } else {
+          if constexpr (q == 0) load_w(WSL{}, c + WD - 1);
+        }
+      };
+      static_for<0, NM>([&](auto m_c) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_c)::value;
+        constexpr int j = m / NFW, f = m % NFW;
+        const u32x4_t wv = wraw[WS4][f][q];
+        // (an fp4 operand is the low four of the eight registers the builtin's type has; the others stay undefined)
+        const i32x8_t a = __builtin_bit_cast(i32x8_t, __builtin_shufflevector(wv, wv, 0, 1, 2, 3, -1, -1, -1, -1));
+        acc[f][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, xf[cur][j], acc[f][j], 4 /* A: e2m1 */, 0 /* B: e4m3 */, q, (int)sdh[f], q,
+                                                                     (int)xs[PAR][j]);
+        if constexpr (q == NS - 1 && m == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        }
+        static_for<(m * NOPS) / NM, ((m + 1) * NOPS) / NM>(op);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+
+  // stage 0 of a unit (every piece, so that the number of loads does not depend on the unit): issued before the
+  // previous unit's epilogue arithmetic
+  auto first_loads = [&]() __attribute__((always_inline)) {
+    static_for<0, XCH>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
+    load_x_scale(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(S0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int up = 0;
+  Unit cur_unit;
+  int resolve_slot = -1;
+  auto run = [&](auto nj_c) __attribute__((always_inline)) {
+    constexpr int NJ = decltype(nj_c)::value;
+    const long long t_run = MX8_T();
+    // the loads left in flight at the loop header are in the order the steady state leaves them in at the top of a
+    // stage: activations, their scales, weights of stage 1, then of stage 2
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
+    store_x_scale(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // what the stages -max(XD, WD - 2) .. -1 would have issued had the loop been running: stage i requests the activations
+    // of stage i + 1 + XD, then the weights of stage i + WD - 1 (this unit's: indices from 1 on)
+    constexpr int LEAD = XD > WD - 2 ? XD : WD - 2;
+    static_for<0, LEAD>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value - LEAD;
+      constexpr int sx = i + 1 + XD, sw = i + WD - 1;
+      if constexpr (sx >= 1) {
+        static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, sx, sx % XD); });
+        load_x_scale(sx, sx % XD);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (sw >= 1) {
+        load_w(template_int<sw % WD>{}, sw);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+    stage_operands(cur_unit, up);
+    if (resolve_slot >= 0 && tid == 0) next_tile_s[resolve_slot] = claimer.resolve();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) {
+      read_xf(0, 0, decltype(jc)::value, xf[0]);
+      read_xs(0, decltype(jc)::value, xs[0]);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    const long long t_loop = MX8_T();
+    MX8_ADD(0, t_loop - t_run);
+    int c = 0;
+    for (; c + UNR - 1 < nst; c += UNR)
+      static_for<0, UNR>([&](auto u_c) __attribute__((always_inline)) { stage(nj_c, u_c, c + decltype(u_c)::value); });
+    static_for<0, UNR - 1>([&](auto u_c) __attribute__((always_inline)) {
+      if (c + decltype(u_c)::value < nst) stage(nj_c, u_c, c + decltype(u_c)::value);
+    });
+    MX8_ADD(1, MX8_T() - t_loop);
+    MX8_ADD(5, nst);
+  };
+
+  const long long t_kernel = MX8_T();
+  if (pid >= 0) {
+    Unit& cur = cur_unit;
+    cur = tile_unit(pid);
+    Unit nxt = advance(cur, pid_next);
+    if (tid < BM) gidx_s[1][tid] = unit_gather_index(cur);
+    __syncthreads();
+    unit_pointers(cur, 1);
+    unit_operands(cur);
+    if (nxt.valid && tid < BM) gidx_v = unit_gather_index(nxt);
+    if (dyn && pid_next >= 0) {
+      claimer.issue();
+      resolve_slot = 0;
+    }
+    first_loads();
+    for (;;) {
+#pragma unroll
+      for (int f = 0; f < NFW; ++f)
+#pragma unroll
+        for (int j = 0; j < MFW; ++j)
+#pragma unroll
+          for (int i = 0; i < FR::NACC; ++i) acc[f][j][i] = 0.f;
+      const int rows = (cur.blk_rows - cur.pass_off) < BM ? (cur.blk_rows - cur.pass_off) : BM;
+      const int nj = (rows + FM - 1) / FM;
+      static_for<1, MFW + 1>([&](auto n_c) __attribute__((always_inline)) {
+        if (nj == decltype(n_c)::value) run(n_c);
+      });
+      resolve_slot = -1;
+      const long long t_prep = MX8_T();
+
+      const int wcol = nw * NFW * FM;
+      const int ncol0 = cur.pid_n * BN + wcol;
+      Unit nxt2 = nxt;
+      if (nxt.valid) {
+        if (cur.pass_off + BM >= cur.blk_rows) {
+          pid = pid_next;
+          ++n_tile;
+          if (dyn) {
+            pid_next = __builtin_amdgcn_readfirstlane(next_tile_s[(n_tile - 1) & 1]);
+          } else {
+            round0 += grid;
+            const int in_round = live - round0 < grid ? live - round0 : grid;
+            pid_next = (int)blockIdx.x < in_round ? round0 + xcd_remap(blockIdx.x, in_round) : -1;
+          }
+          if (dyn && pid_next >= 0) {
+            claimer.issue();
+            resolve_slot = n_tile & 1;
+          }
+        }
+        nxt2 = advance(nxt, pid_next);
+        unit_operands(nxt);
+        if (nxt2.valid && tid < BM) gidx_v = unit_gather_index(nxt2);
+        __builtin_amdgcn_sched_barrier(0);
+        unit_pointers(nxt, up);
+        first_loads();
+      }
+      const long long t_epi = MX8_T();
+      MX8_ADD(2, t_epi - t_prep);
+      if constexpr (MXOUT)
+        staged_mx_epilogue<MFW, NFW, SWIGLU>(p, acc, yrsrc, ysrsrc, bias_s[up], gam_s[up], dst_s[up], wcol, ncol0, lr, h);
+      else
+        staged_epilogue<1, MFW, NFW, NFW, SWIGLU, true>(p, acc, yrsrc, bias_s[up], gam_s[up], dst_s[up], wcol, ncol0, 0, lr, h);
+      MX8_ADD(3, MX8_T() - t_epi);
+      MX8_ADD(4, 1);
+      if (!nxt.valid) break;
+      cur = nxt;
+      nxt = nxt2;
+      up ^= 1;
+    }
+  }
+  if (dyn) claimer.finish();
+  MX8_ADD(6, MX8_T() - t_kernel);
+}
+
 template <int BLKM, int MFW, int NFW>
 int32_t launch_mx8n(const GemmParams& p, int grid_m, bool swiglu, bool mxout, hipStream_t st) {
   constexpr int LDS_BYTES = 2 * MFW * 32 * (128 + 16);
@@ -443,6 +986,13 @@ int32_t launch_mx8n(const GemmParams& p, int grid_m, bool swiglu, bool mxout, hi
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS_BYTES, st, q);
     return check_launch("moe_gemm_mx8n_kernel");
   };
+  if (p.y_bytes != 0) {
+    // (the host found what the persistent form needs)
+    if (swiglu && mxout) return launch(moe_gemm_mx8p_kernel<BLKM, MFW, NFW, true, true>);
+    if (swiglu) return launch(moe_gemm_mx8p_kernel<BLKM, MFW, NFW, true, false>);
+    if (mxout) return launch(moe_gemm_mx8p_kernel<BLKM, MFW, NFW, false, true>);
+    return launch(moe_gemm_mx8p_kernel<BLKM, MFW, NFW, false, false>);
+  }
   if (swiglu && mxout) return launch(moe_gemm_mx8n_kernel<BLKM, MFW, NFW, true, true>);
   if (swiglu) return launch(moe_gemm_mx8n_kernel<BLKM, MFW, NFW, true, false>);
   if (mxout) return launch(moe_gemm_mx8n_kernel<BLKM, MFW, NFW, false, true>);
@@ -450,6 +1000,16 @@ int32_t launch_mx8n(const GemmParams& p, int grid_m, bool swiglu, bool mxout, hi
 }
 
 }  // namespace
+
+#ifdef TK_MX8_STAMPS
+extern "C" int32_t tk_debug_mx8_stamps(long long* host_out, int32_t clear) {
+  if (clear) {
+    static long long zeros[1024 * 8];
+    return hipMemcpyToSymbol(HIP_SYMBOL(mx8_stamps), zeros, sizeof(zeros)) == hipSuccess ? 0 : 3;
+  }
+  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(mx8_stamps), sizeof(long long) * 1024 * 8) == hipSuccess ? 0 : 3;
+}
+#endif
 
 int32_t gemm_launch_mx8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, bool mx_out, hipStream_t st) {
   //                                       BLKM MFW NFW

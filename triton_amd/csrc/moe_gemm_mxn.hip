@@ -32,76 +32,6 @@ namespace {
 // BM = 32 * MFW * G rows; with BLKM = 256 and MFW = 5 an expert of up to 160 rows is ONE tile (weights read
 // once, no nearly empty second tile) and only larger blocks take a second pass.
 
-// Epilogue of the persistent prefill kernels.  Everything a tile's rows and columns need (bias as fp32, gate weight,
-// destination row or -1) was fetched ahead and sits in LDS: bias_s[BN] by tile column, gam_s / dst_s [BM] by tile
-// row.  Order: bias, activation, gate weight, (scattered) store.  The bias is added as each accumulator register
-// is read for the last time (a pass of its own over the accumulators would move all of them between the
-// accumulation and the vector registers twice more).
-// Every lane executes every store instruction: rows without a destination and columns past N get a byte offset
-// beyond the buffer resource's range, which the hardware drops.  With no branch around a store the number of
-// stores between two loads is the same on every path, so the compiler's vmcnt waits for loads issued BEFORE the
-// epilogue (the next unit's first operands) do not wait for these stores to drain.
-
-// NFV = leading column fragments of the wave that hold real columns; the others skip the arithmetic and issue their
-// stores with the dropped offset, so that the number of stores is the same on every path.
-template <int G, int MFW, int NFW, int NFV, bool SWIGLU>
-__device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc, const float* bias_s,
-                                                const float* gam_s, const int* dst_s, int ncol_tile, int ncol0, int grp, int lr, int h) {
-  const int NOUT = SWIGLU ? p.N / 2 : p.N;
-  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
-  const float limit = p.has_limit ? p.limit : INFINITY;
-  const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
-#pragma unroll
-  for (int j = 0; j < MFW; ++j) {
-    const int r = (j * G + grp) * 32 + lr;
-    const float g = gam_s[r];
-    const int dst = dst_s[r];
-    const uint32_t row_off = dst >= 0 ? (uint32_t)dst * row_bytes : kDroppedStore;
-#pragma unroll
-    for (int f = 0; f < NFW; ++f)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        if (f >= NFV) {
-          if (SWIGLU)
-            __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{0u, 0u}, yrsrc, kDroppedStore, 0, 0);
-          else
-            __builtin_amdgcn_raw_buffer_store_b128(u32x4_t{0u, 0u, 0u, 0u}, yrsrc, kDroppedStore, 0, 0);
-          continue;
-        }
-        // registers 8u..8u+3 hold columns 16u + 4h + i, registers 8u+4..8u+7 columns 16u + 8 + 4h + i: after the two
-        // lane halves exchange their 4-column groups a lane holds 8 consecutive columns from 16u + 8h
-        float v[8];
-        // bias of the two column groups (zeros without a bias), re-read from LDS for every row fragment: keeping all
-        // of a lane's 32 bias values in registers costs more than the reads
-        const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 4 * h);
-        const f32x4_t b1 = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 8 + 4 * h);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          uint32_t lo = f32_bits(acc[f][j][8 * u + i] + b0[i]), hi = f32_bits(acc[f][j][8 * u + 4 + i] + b1[i]);
-          auto sw = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);
-          v[i] = bits_f32(sw[0]);
-          v[4 + i] = bits_f32(sw[1]);
-        }
-        const int n0 = ncol0 + f * 32 + 16 * u + 8 * h;  // first of this lane's 8 columns
-        if (SWIGLU) {
-          float o[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) o[i] = swiglu_f(v[2 * i], v[2 * i + 1], nalpha_log2e, limit) * g;
-          const int o0 = n0 / 2;
-          const uint32_t off = (o0 < NOUT && dst >= 0) ? row_off + (uint32_t)o0 * 2u : kDroppedStore;
-          const u32x2_t w = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
-          __builtin_amdgcn_raw_buffer_store_b64(w, yrsrc, off, 0, 0);
-        } else {
-          const uint32_t off = (n0 < NOUT && dst >= 0) ? row_off + (uint32_t)n0 * 2u : kDroppedStore;
-          u32x4_t w;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i] * g, v[2 * i + 1] * g);
-          __builtin_amdgcn_raw_buffer_store_b128(w, yrsrc, off, 0, 0);
-        }
-      }
-  }
-}
-
 template <int BLKM, int MFW, int NFW, int G, int WD, int XD, bool SWIGLU>
 __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams p) {
   typedef Frag<32> FR;
@@ -582,83 +512,8 @@ __global__ __launch_bounds__(256 * G) void moe_gemm_mxn_kernel(const GemmParams 
     }
   }
   if (dyn) claimer.finish();
-  // ---- top-k combine behind the scatter (reduce.py:1143-1165 after matmul_details/_matmul.py:535-569 in the reference,
-  // a launch of its own there): out[t, :] = sum over j of y[t * k + j, :], fp32 in j order, bf16 result.  The k rows of a
-  // token come from k experts, i.e. from tiles of workgroups all over the chip, so the sum runs when EVERY workgroup
-  // has written its tiles: the grid is persistent and fits the GPU (one workgroup per CU).
-  //   1. a workgroup whose stores have all reached its XCD's L2 counts itself in (per XCD and in total);
-  //   2. when all have, ONE workgroup per XCD (the first to claim it) has that L2 write its dirty lines back (a release
-  //      fence; one per L2, not one per wave: every fence walks the whole cache) and reports it;
-  //   3. when every XCD in use has reported, the rows of y are in memory: the workgroups sum the tokens blockIdx.x,
-  //      blockIdx.x + grid, ..., reading y around their own L2 (sc0 sc1: lines another XCD wrote are not coherent in it);
-  //   4. the last workgroup to leave clears the words for the next launch.
-  // Words of `tile_counters`: 9 arrivals, 10 departures, 11 error (raised, and kept, if a bounded wait runs out),
-  // 12 XCDs in use, 13 XCDs written back, 16..23 arrivals per XCD, 24..31 write-back claimed per XCD.
   if constexpr (!SWIGLU) {
-    if (p.combine_k > 0 && p.tile_counters != nullptr) {
-      int32_t* ctr = p.tile_counters;
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      if (tid == 0) {
-        int xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        xcc &= 7;
-        auto wait_for = [&](int32_t* word, int want) {
-          int spins = 0;
-          while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
-            __builtin_amdgcn_s_sleep(16);
-            if (++spins > (1 << 22)) {
-              atomicOr(&ctr[11], 1);
-              break;
-            }
-          }
-        };
-        if (__hip_atomic_fetch_add(&ctr[16 + xcc], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
-          __hip_atomic_fetch_add(&ctr[12], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_fetch_add(&ctr[9], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        wait_for(&ctr[9], grid);
-        if (__hip_atomic_fetch_add(&ctr[24 + xcc], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this XCD's L2 writes back its dirty lines
-          __hip_atomic_fetch_add(&ctr[13], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        wait_for(&ctr[13], __hip_atomic_load(&ctr[12], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      }
-      __syncthreads();
-      const int k = p.combine_k, T = p.scatter_len / k;
-      const int n8 = N >> 3;  // (N is a multiple of 8: host check)
-      const __amdgpu_buffer_rsrc_t ysrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
-      const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
-      constexpr int kAround = 1 | 16;  // sc0 | sc1
-      for (int t = blockIdx.x; t < T; t += grid) {
-        for (int c = tid; c < n8; c += NT) {
-          float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          for (int j0 = 0; j0 < k; j0 += 4) {
-            u32x4_t v[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const uint32_t off = j0 + q < k ? (uint32_t)(t * k + j0 + q) * row_bytes + (uint32_t)c * 16u : kDroppedStore;
-              v[q] = __builtin_amdgcn_raw_buffer_load_b128(ysrc, off, 0, kAround);  // (dropped offsets read zero)
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                sum[2 * e] += bits_f32(v[q][e] << 16);
-                sum[2 * e + 1] += bits_f32(v[q][e] & 0xFFFF0000u);
-              }
-          }
-          *reinterpret_cast<u32x4_t*>(p.combine_out + (int64_t)t * p.combine_stride + c * 8) =
-              u32x4_t{pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]), pack_bf16x2(sum[4], sum[5]), pack_bf16x2(sum[6], sum[7])};
-        }
-      }
-      __syncthreads();
-      if (tid == 0) {
-        if (__hip_atomic_fetch_add(&ctr[10], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == grid - 1) {
-          for (int w = 9; w < 32; ++w)
-            if (w != 11) __hip_atomic_store(&ctr[w], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      }
-    }
+    if (p.combine_k > 0 && p.tile_counters != nullptr) fused_prefill_combine<NT>(p, tid, grid);
   }
 }
 

@@ -783,6 +783,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     if (tiled or tiled_fp8) and block_m >= 64 and not _STATIC_TILES and not mx_act:
         d.tile_counters = _tile_counters(a.device).data_ptr()
     combined = None
+    # (not with MXFP8 activations: at the end of that kernel's launch the combine measured 22 us slower than `reduce` in a
+    # launch of its own at the gpt-oss shape)
     can_combine = (_combine_k and not extras and tiled and not mx_act and act == nt.TK_ACT_NONE and scatter_indx is not None
                    and scatter_indx.shape[0] % _combine_k == 0 and a.dtype == torch.bfloat16)
     if can_combine and block_m <= 32:
