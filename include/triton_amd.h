@@ -287,7 +287,7 @@ typedef struct tk_gemm_desc {
   int32_t M, N, K; /* M: rows of the single slice when not ragged; N: columns of W; K: reduction */
   /* output [rows, N or N/2], unit stride along N */
   void* y;
-  int32_t y_dtype; /* TK_BF16, TK_F16 (fp16 operands), or TK_E4M3 with y_mx_scale */
+  int32_t y_dtype; /* TK_BF16, TK_F16 (fp16 operands), or with y_mx_scale TK_E4M3 / TK_E5M2 / TK_E2M1 (see there) */
   int64_t y_stride_m;
   int32_t activation; /* enum tk_activation */
   float act_alpha, act_limit;
@@ -313,10 +313,14 @@ typedef struct tk_gemm_desc {
    * storage formats. */
   const void* x_mx_scale;
   int64_t xs_stride_m;
-  /* MX-quantised output (y_dtype TK_E4M3, MXFP8-activation path only): the epilogue quantises the fp32 accumulator,
-   * after bias, activation and gate weight, in blocks of 32 output columns (the `QUANTIZE_MXFP8` epilogue,
-   * tk/matmul_details/_matmul.py:593-637): e4m3 bytes to y, one e8m0 byte per block to y_mx_scale
-   * [rows of y, N_out / 32].  NULL = plain bf16 output. */
+  /* MX-quantised output: the epilogue quantises the fp32 accumulator, after bias, activation and gate weight, in blocks
+   * of 32 output columns (the `QUANTIZE_MXFP8` / `QUANTIZE_MXFP4` epilogues, tk/matmul_details/_matmul.py:593-637):
+   * values to y, one e8m0 byte per block (round-up rule) to y_mx_scale [rows of y, N_out / 32]; N_out % 32 == 0.
+   *   MXFP8 activations (x_mx_scale):                                 y_dtype TK_E4M3
+   *   bf16 activations, tiled MXFP4 weights, block_m 128 or 256:      y_dtype TK_E4M3, TK_E5M2 or TK_E2M1 (two codes per byte,
+   *     even column in the low nibble; y_stride_m then counts bytes); rows of y 8-byte aligned; not with betas /
+   *     out_alpha / acc_in or the fused combine
+   * NULL = plain bf16 output.  Other operand combinations quantise in a second pass (tk_mx_downcast on the bf16 result). */
   void* y_mx_scale;
   int64_t ys_stride_m;
   /* Fused top-k combine behind the scatter (bf16 activations, tiled MXFP4 weights, no activation).  At block_m >= 64

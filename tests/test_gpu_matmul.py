@@ -333,8 +333,10 @@ def test_fused_swiglu(mods, device, m, n, k, wkind, block_m, opts):
 def test_mx_output_epilogue(mods, device, kind, wkind, swiglu, scatter):
     """`Epilogue(FnSpecs(QUANTIZE_MXFP8 | QUANTIZE_MXFP4))` + `c_mx_scale` (reference test: tests/test_matmul.py:560-573,
     checked at :627-643 by dequantising and comparing with maxtol 4e-1 / rmstol 4e-2 against the quantised reference).
-    Two checks: (1) the values and scales are bit for bit the oracle's quantisation of the GEMM's own bf16 output;
-    (2) dequantised, they meet the reference's tolerance against the oracle's GEMM -> quantise -> dequantise."""
+    Strided weights run the bf16 GEMM followed by the MX quantiser kernel: (1) the values and scales are bit for bit the
+    oracle's quantisation of the GEMM's own bf16 output; (2) dequantised, they meet the reference's tolerance against the
+    oracle's GEMM -> quantise -> dequantise.  Tiled MXFP4 weights quantise the fp32 accumulator inside the GEMM and are
+    checked against the oracle's fp32 GEMM -> oracle quantiser in `test_bf16_activations_with_fused_mx_output`."""
     mm, sw, tensor = mods
     from triton_amd.numerics_details.mxfp import quantize_mxfp4_fn, quantize_mxfp8_fn
     g = torch.Generator().manual_seed(17)
@@ -355,11 +357,13 @@ def test_mx_output_epilogue(mods, device, kind, wkind, swiglu, scatter):
     pc = mm.PrecisionConfig(b_mx_scale=W["scale_dev"], c_mx_scale=c_scale, out_dtype=out_dtype)
     yq = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=pc, epilogue=epi, **kw)
     assert yq.dtype == out_dtype and yq.shape == (m, n_out // 2 if kind == "mxfp4" else n_out)
-    assert pc.c_mx_scale is c_scale and pc.c_value_pack_factor == (2 if kind == "mxfp4" else 1)
-    y = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]), **kw)
-    q_ref, s_ref = omx.downcast_to_mxfp(y.cpu(), out_dtype, axis=-1)
-    assert torch.equal(q_ref.view(torch.uint8), yq.cpu().view(torch.uint8)), "values are not the quantisation of the bf16 result"
-    assert torch.equal(s_ref, c_scale.cpu()), "scales are not the quantisation of the bf16 result"
+    # the caller's PrecisionConfig is left as it was given (the reference records the pack factor on it, matmul.py:364-369)
+    assert pc.c_mx_scale is c_scale and pc.c_value_pack_factor == 1 and pc.c_microblock_size is None
+    if wkind != "mxfp4_tiled":
+        y = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=mm.PrecisionConfig(b_mx_scale=W["scale_dev"]), **kw)
+        q_ref, s_ref = omx.downcast_to_mxfp(y.cpu(), out_dtype, axis=-1)
+        assert torch.equal(q_ref.view(torch.uint8), yq.cpu().view(torch.uint8)), "values are not the quantisation of the bf16 result"
+        assert torch.equal(s_ref, c_scale.cpu()), "scales are not the quantisation of the bf16 result"
     h = omoe.matmul(x, W["w_cpu"], bias, sizes, w_mx_scale=W["scale_cpu"], scatter_indx=sc)
     if swiglu:
         h = omoe.swiglu(h, 1.702, 7.0)
@@ -666,6 +670,67 @@ def test_mxfp8_activations_with_fused_mx_output(mods, device, swiglu, scatter, b
     assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
     # the quantised result is close to the unquantised GEMM (e4m3 has 3 mantissa bits: half a step is 2^-4 relative)
     assert_close(h, got, maxtol=1.0, rmstol=4e-2, what="MX output against the unquantised result")
+
+
+@pytest.mark.parametrize("kind", ["mxfp8_e4m3", "mxfp8_e5m2", "mxfp4"])
+@pytest.mark.parametrize("swiglu, scatter, gamma", [(True, False, False), (False, True, True), (False, False, False)])
+@pytest.mark.parametrize("block_m", [128, 256])
+def test_bf16_activations_with_fused_mx_output(mods, device, monkeypatch, kind, swiglu, scatter, gamma, block_m):
+    """bf16 activations x tiled MXFP4 weights with `Epilogue(QUANTIZE_MXFP8 | QUANTIZE_MXFP4)`: the prefill kernel's epilogue
+    quantises the fp32 accumulator (matmul_details/_matmul.py:593-637) to e4m3, e5m2 or packed e2m1.  Against the oracle's
+    GEMM (fp32 result, bias, swiglu, gate weight) -> oracle MX quantiser: block scales equal except where the two fp32
+    sums put a block's maximum on different sides of a power-of-two boundary, nearly all codes bit-equal, and the
+    dequantised values within the reference's tolerance for this epilogue (tests/test_matmul.py:627-643)."""
+    mm, sw_mod, tensor = mods
+    from triton_amd.numerics_details.mxfp import quantize_mxfp4_fn, quantize_mxfp8_fn
+    g = torch.Generator().manual_seed(29 + block_m)
+    m, n, k, n_slices = 700, 640, 416, 6
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    W = _make_w(n_slices, k, n, "mxfp4_tiled", g, device)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = _slice_sizes(m, n_slices, g)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    sc = torch.randperm(m, generator=g).to(torch.int32) if scatter else None
+    gammas = 2.0**torch.randint(-5, 0, (m, ), generator=g).float() if gamma else None
+    act = mm.FusedActivation(mm.FnSpecs("swiglu", sw_mod.swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if swiglu else None
+    n_out = n // 2 if swiglu else n
+    out_dtype = {"mxfp8_e4m3": torch.float8_e4m3fn, "mxfp8_e5m2": torch.float8_e5m2, "mxfp4": torch.uint8}[kind]
+    name, fn = (mm.FnName.QUANTIZE_MXFP4.name, quantize_mxfp4_fn) if kind == "mxfp4" else (mm.FnName.QUANTIZE_MXFP8.name, quantize_mxfp8_fn)
+    epi = mm.Epilogue(mm.FnSpecs(name, fn, (), ()), tuple(), tuple(), effective_itemsize=6.0)
+    c_scale = torch.full((m, n_out // 32), 0xFF, dtype=torch.uint8, device=device)
+    pc = mm.PrecisionConfig(b_mx_scale=W["scale_dev"], c_mx_scale=c_scale, out_dtype=out_dtype)
+    def two_step(*args, **kwargs):
+        raise AssertionError("the GEMM + quantiser path ran instead of the fused epilogue")
+
+    monkeypatch.setattr(mm, "_matmul_mx_out", two_step)
+    with mm.scoped_opt_flags_constraints({"block_m": block_m}):
+        yq = mm.matmul(x.to(device), W["w_dev"], bias.to(device), md, precision_config=pc, epilogue=epi, fused_activation=act,
+                       scatter_indx=None if sc is None else sc.to(device), gammas=None if gammas is None else gammas.to(device))
+    assert yq.dtype == out_dtype and yq.shape == (m, n_out // 2 if kind == "mxfp4" else n_out)
+    h = omoe.matmul(x, W["w_cpu"], bias, sizes, w_mx_scale=W["scale_cpu"], scatter_indx=sc, gammas=None if swiglu else gammas, out_dtype=torch.float32)
+    if swiglu:
+        h = omoe.swiglu(h, 1.702, 7.0)
+    q_ref, s_ref = omx.downcast_to_mxfp(h, out_dtype, axis=-1)
+    s_got, q_got = c_scale.cpu(), yq.cpu()
+    scale_diff = (s_ref != s_got).float().mean().item()
+    assert scale_diff <= 2e-3, f"{scale_diff:.4g} of the block scales differ from the oracle's"
+    if kind == "mxfp4":
+        lo_diff = ((q_ref & 0xF) != (q_got & 0xF)).float().mean().item()
+        hi_diff = ((q_ref >> 4) != (q_got >> 4)).float().mean().item()
+        code_diff = 0.5 * (lo_diff + hi_diff)
+    else:
+        code_diff = (q_ref.view(torch.uint8) != q_got.view(torch.uint8)).float().mean().item()
+    assert code_diff <= 0.02, f"{code_diff:.4g} of the {kind} codes differ from the oracle's"
+    ref = omx.upcast_from_mxfp(q_ref, s_ref, torch.bfloat16, axis=-1)
+    got = omx.upcast_from_mxfp(q_got, s_got, torch.bfloat16, axis=-1)
+    if kind == "mxfp4":
+        # 3-bit magnitudes: a code that differs moves a value by a whole e2m1 step, so the bound is on how many differ (above)
+        # and on the rms error
+        from oracle.checks import rel_errors
+        _, rms = rel_errors(ref, got)
+        assert rms <= 3e-2, f"mxfp4 output: rms {rms:.4g}"
+    else:
+        assert_close(ref, got, maxtol=4e-1, rmstol=4e-2, what="dequantised MX output")
 
 
 @pytest.mark.parametrize("kind", ["bf16", "mxfp4", "mxfp4_tiled"])

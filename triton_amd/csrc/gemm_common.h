@@ -60,8 +60,9 @@ struct GemmParams {
   int32_t* combine_counters;  // zeroed [tokens * ceil(N / 32)] words, left zero
   const uint8_t* x_mx_scale;  // e8m0 block scales of MXFP8 activations [rows, K/32], or null
   int64_t xs_stride_m;
-  uint8_t* y_mx_scale;        // e8m0 block scales of an MXFP8 output [rows, N_out/32], or null
+  uint8_t* y_mx_scale;        // e8m0 block scales of an MX-quantised output [rows, N_out/32], or null
   int64_t ys_stride_m;
+  int32_t y_mx_kind;          // TK_E4M3, TK_E5M2 or TK_E2M1: the element type of an MX-quantised output
   // options of the shared epilogue only (the host keeps them away from the kernels with an epilogue of their own)
   const void* betas;          // per expert-sorted row multiplier of the bias, or null
   int32_t betas_is_f32;
@@ -74,6 +75,7 @@ struct GemmParams {
 // one entry per kernel family; each returns a TK_* status
 int32_t gemm_launch_strided(const GemmParams& p, int wk, int block_m, int grid_m, bool swiglu, hipStream_t st);
 int32_t gemm_launch_mxn(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_mxn_mx(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);  // block_m 128 / 256, MX-quantised output
 int32_t gemm_launch_mxd(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
 int32_t gemm_launch_f8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
 int32_t gemm_launch_mx8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, bool mx_out, hipStream_t st);
@@ -605,6 +607,141 @@ __device__ __forceinline__ void staged_epilogue(const GemmParams& p, f32x16_t (&
           __builtin_amdgcn_raw_buffer_store_b128(w, yrsrc, off, 0, 0);
         }
       }
+  }
+}
+
+
+// MX-quantised output of the persistent prefill kernels (matmul_details/_matmul.py:593-637): blocks of 32 output columns of the
+// fp32 accumulator (after bias, activation and gate weight), one e8m0 scale byte per block (round-up rule) to y_mx_scale, values
+// as e4m3, e5m2 or packed e2m1 (p.y_mx_kind) to y.  The operands of rows and columns are taken
+// from LDS (bias_s by tile column, gam_s / dst_s by tile row, fetched a unit ahead) and with no branch around a store:
+// rows without a destination, columns past the end and the lanes that do not write a block's scale byte store to an
+// offset beyond the range of their buffer resource, which the hardware drops.
+template <int MFW, int NFW, bool SWIGLU>
+__device__ __forceinline__ void staged_mx_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc,
+                                                   __amdgpu_buffer_rsrc_t ysrsrc, const float* bias_s, const float* gam_s, const int* dst_s,
+                                                   int ncol_tile, int ncol0, int lr, int h) {
+  const int NOUT = SWIGLU ? p.N / 2 : p.N;
+  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
+  const float limit = p.has_limit ? p.limit : INFINITY;
+  constexpr int VO = SWIGLU ? 4 : 8;
+  constexpr int NB = SWIGLU ? 1 : NFW;
+  // every LDS operand up front: one round trip for the unit
+  f32x4_t bh[NFW][2][2];
+  float gh[MFW];
+  int dh[MFW];
+#pragma unroll
+  for (int f = 0; f < NFW; ++f)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      bh[f][u][0] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 4 * h);
+      bh[f][u][1] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 8 + 4 * h);
+    }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    gh[j] = gam_s[j * 32 + lr];
+    dh[j] = dst_s[j * 32 + lr];
+  }
+#pragma unroll
+  for (int j = 0; j < MFW; ++j) {
+    const float g = gh[j];
+    const int dst = dh[j];
+    float o[NFW][2][VO];
+#pragma unroll
+    for (int f = 0; f < NFW; ++f)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(acc[f][j][8 * u + i] + bh[f][u][0][i]), f32_bits(acc[f][j][8 * u + 4 + i] + bh[f][u][1][i]), false, false);
+          v[i] = bits_f32(sw[0]);
+          v[4 + i] = bits_f32(sw[1]);
+        }
+#pragma unroll
+        for (int i = 0; i < VO; ++i) o[f][u][i] = SWIGLU ? swiglu_f(v[2 * i], v[2 * i + 1], nalpha_log2e, limit) * g : v[i] * g;
+      }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      // block maximum of |o|: fmaxf returns its other operand for a NaN, so a NaN never wins and the block's scale comes
+      // from its finite values.  (N_out is a multiple of 32: a block lies below it whole or not at all, and one that does
+      // not is not stored.)
+      float m = 0.f;
+#pragma unroll
+      for (int f = 0; f < NFW; ++f) {
+        if (!SWIGLU && f != b) continue;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < VO; ++i) m = __builtin_fmaxf(m, __builtin_fabsf(o[f][u][i]));
+      }
+      {
+        // the other lane half's maximum: after the swap the first register holds both halves' lanes 0..31, the second both
+        // halves' lanes 32..63
+        auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(m), f32_bits(m), false, false);
+        m = __builtin_fmaxf(bits_f32(sw[0]), bits_f32(sw[1]));
+      }
+      const int kind = p.y_mx_kind;  // uniform
+      const uint32_t sbits = mx_scale_bits(m, kind, TK_MX_ROUND_UP);
+      const float inv = mx_inv_scale(sbits);
+      const int blk_col0 = SWIGLU ? ncol0 / 2 : ncol0 + b * 32;
+      const uint32_t soff = (dst >= 0 && h == 0 && blk_col0 < NOUT) ? (uint32_t)dst * (uint32_t)p.ys_stride_m + (uint32_t)(blk_col0 >> 5) : kDroppedStore;
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(sbits >> 23), ysrsrc, soff, 0, 0);
+#pragma unroll
+      for (int f = 0; f < NFW; ++f) {
+        if (!SWIGLU && f != b) continue;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int col0 = SWIGLU ? (ncol0 + f * 32 + 16 * u + 8 * h) / 2 : ncol0 + f * 32 + 16 * u + 8 * h;
+          // No clamp in front of the conversion: the scale is the smallest power of two >= max / max_q (the rounded quotient
+          // of an fp32 by 448 = 1.75 * 2^8, 57344 = 1.75 * 2^15 or 6 = 1.5 * 2^2 is a power of two only when the exact one
+          // is), scaling by a power of two is exact, so |o * inv| <= max_q for every finite block; with an infinite maximum
+          // inv is 0.  The three kinds issue the same number of stores (the wait counts of loads issued ahead stay exact).
+          float qv[VO];
+#pragma unroll
+          for (int i = 0; i < VO; ++i) qv[i] = o[f][u][i] * inv;
+          const bool live = dst >= 0 && col0 < NOUT;
+          if (kind == TK_E2M1) {
+            // two codes per byte, even column in the low nibble; NaN saturates like the infinity of its sign (mxfp.py:298-327)
+#pragma unroll
+            for (int i = 0; i < VO; ++i) qv[i] = qv[i] != qv[i] ? __builtin_copysignf(INFINITY, qv[i]) : qv[i];
+            uint32_t w = 0;
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, qv[0], qv[1], 1.0f, 0);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, qv[2], qv[3], 1.0f, 1);
+            const uint32_t off = live ? (uint32_t)dst * (uint32_t)p.y_stride_m + (uint32_t)(col0 >> 1) : kDroppedStore;
+            if constexpr (VO == 8) {
+              w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, qv[4], qv[5], 1.0f, 2);
+              w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, qv[6], qv[7], 1.0f, 3);
+              __builtin_amdgcn_raw_buffer_store_b32(w, yrsrc, off, 0, 0);
+            } else {
+              __builtin_amdgcn_raw_buffer_store_b16((uint16_t)w, yrsrc, off, 0, 0);
+            }
+          } else {
+            const uint32_t off = live ? (uint32_t)dst * (uint32_t)p.y_stride_m + (uint32_t)col0 : kDroppedStore;
+            int w0 = 0, w1 = 0;
+            if (kind == TK_E4M3) {
+              w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[0], qv[1], w0, false);
+              w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[2], qv[3], w0, true);
+              if constexpr (VO == 8) {
+                w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[4], qv[5], w1, false);
+                w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[6], qv[7], w1, true);
+              }
+            } else {
+              w0 = __builtin_amdgcn_cvt_pk_bf8_f32(qv[0], qv[1], w0, false);
+              w0 = __builtin_amdgcn_cvt_pk_bf8_f32(qv[2], qv[3], w0, true);
+              if constexpr (VO == 8) {
+                w1 = __builtin_amdgcn_cvt_pk_bf8_f32(qv[4], qv[5], w1, false);
+                w1 = __builtin_amdgcn_cvt_pk_bf8_f32(qv[6], qv[7], w1, true);
+              }
+            }
+            if constexpr (VO == 8)
+              __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{(uint32_t)w0, (uint32_t)w1}, yrsrc, off, 0, 0);
+            else
+              __builtin_amdgcn_raw_buffer_store_b32((uint32_t)w0, yrsrc, off, 0, 0);
+          }
+        }
+      }
+    }
   }
 }
 

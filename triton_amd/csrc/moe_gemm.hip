@@ -19,8 +19,12 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   if (d->x_dtype != TK_BF16 && d->x_dtype != TK_E4M3 && !f16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations must be bf16, fp16 or e4m3 (dtype %d)", d->x_dtype);
   const bool mx_act = d->x_dtype == TK_E4M3 && d->x_mx_scale != nullptr;  // MXFP8 activations: scaled-MFMA path
   if (!mx_act && (d->x_dtype == TK_E4M3) != (d->w_dtype == TK_E4M3)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: e4m3 activations go with e4m3 weights, or with MX scales and tiled MXFP4 weights (x dtype %d, w dtype %d)", d->x_dtype, d->w_dtype);
-  const bool mx_out = d->y_dtype == TK_E4M3 && d->y_mx_scale != nullptr;
-  if (d->y_dtype != TK_BF16 && !f16 && !(mx_out && mx_act)) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16, or e4m3 with y_mx_scale on the MXFP8-activation path (dtype %d)", d->y_dtype);
+  // MX-quantised output from the fp32 accumulator: e4m3 on the MXFP8-activation path; e4m3 / e5m2 / packed e2m1 with bf16
+  // activations and tiled MXFP4 weights at block_m 128 / 256
+  const bool mx_out = d->y_mx_scale != nullptr && (d->y_dtype == TK_E4M3 || (!mx_act && (d->y_dtype == TK_E5M2 || d->y_dtype == TK_E2M1)));
+  const bool mx_out_bf16 = mx_out && !mx_act && d->x_dtype == TK_BF16 && d->w_layout == TK_W_TILED && d->w_dtype == TK_E2M1 && (d->block_m == 128 || d->block_m == 256);
+  if (d->y_dtype != TK_BF16 && !f16 && !(mx_out && (mx_act || mx_out_bf16)))
+    return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: output must be bf16, or MX-quantised (y_mx_scale): e4m3 with MXFP8 activations; e4m3, e5m2 or e2m1 with bf16 activations and tiled MXFP4 weights at block_m 128 / 256 (dtype %d)", d->y_dtype);
   if (d->activation != TK_ACT_NONE && d->activation != TK_ACT_SWIGLU) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad activation %d", d->activation);
   if (d->activation == TK_ACT_SWIGLU && d->N % 2) return fail(TK_ERR_INVALID, "tk_moe_gemm: swiglu needs an even N");
   const int xe = d->x_dtype == TK_E4M3 ? 16 : 8;  // elements per 16 bytes
@@ -105,6 +109,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
   p.xs_stride_m = d->xs_stride_m;
   p.y_mx_scale = static_cast<uint8_t*>(d->y_mx_scale);
   p.ys_stride_m = d->ys_stride_m;
+  p.y_mx_kind = d->y_dtype;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool swiglu = d->activation == TK_ACT_SWIGLU;
   if (d->w_layout == TK_W_TILED && d->w_dtype == TK_E4M3) {
@@ -158,6 +163,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->w_dtype != TK_E2M1 || !d->w_mx_scale || d->x_dtype != TK_BF16) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the tiled weight layout holds MXFP4 weights for bf16 activations");
     if (d->block_m != 16 && d->block_m != 32 && d->block_m != 64 && d->block_m != 128 && d->block_m != 256) return fail(TK_ERR_INVALID, "tk_moe_gemm: block_m must be 16, 32, 64, 128 or 256 (got %d)", d->block_m);
     if (d->block_m >= 64 && extras) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: betas / out_alpha / acc_in need block_m 16 or 32 with tiled MXFP4 weights");
+    if (mx_out_bf16 && d->combine_k > 0) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: the fused top-k combine needs a bf16 output");
     if (d->block_m >= 64) {
       // the prefill kernels address activation rows with 32-bit byte offsets from x
       if (d->gather_indx && d->x_rows <= 0)
@@ -166,7 +172,19 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
       if (d->x_stride_m * 2 >= (int64_t)1 << 32 || rows * d->x_stride_m * 2 > (int64_t)1 << 32)
         return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: activations of 4 GiB and more are not supported with tiled MXFP4 weights (%lld rows, row stride %lld)", (long long)rows, (long long)d->x_stride_m);
     }
-    if (d->block_m >= 64) {
+    if (mx_out_bf16) {
+      // y_stride_m counts stored elements: bytes, two e2m1 codes each for TK_E2M1.  A lane stores the 4 (swiglu) or 8 values
+      // of its column group in one piece of 2 to 8 bytes.
+      const int64_t n_out = swiglu ? d->N / 2 : d->N;
+      const int64_t y_rows = d->scatter_indx ? d->scatter_len : d->M;
+      const int64_t row_bytes = d->y_dtype == TK_E2M1 ? n_out / 2 : n_out;
+      const int64_t y_bytes = y_rows * d->y_stride_m;
+      if (n_out % 32) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: an MX-quantised output needs N_out %% 32 == 0 (got %lld)", (long long)n_out);
+      if (d->y_stride_m % 8 || (reinterpret_cast<uintptr_t>(d->y) & 7) || d->y_stride_m < row_bytes || d->ys_stride_m < n_out / 32)
+        return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: rows of an MX-quantised output must be 8-byte aligned and hold the row (row stride %lld for %lld bytes)", (long long)d->y_stride_m, (long long)row_bytes);
+      if (y_bytes >= (int64_t)1 << 31 || y_rows * d->ys_stride_m >= (int64_t)1 << 31) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: outputs of 2 GiB and more are not supported with tiled MXFP4 weights");
+      p.y_bytes = (uint32_t)y_bytes;
+    } else if (d->block_m >= 64) {
       // the prefill kernels store through a buffer resource with 16-byte (8-byte with swiglu) pieces per lane: rows
       // must be 16-byte aligned and long enough to take the last piece whole
       const int64_t n_out = swiglu ? d->N / 2 : d->N;
@@ -186,6 +204,7 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
     if (d->block_m <= 32) return gemm_launch_mxd(p, d->block_m, d->grid_m, swiglu, st);
+    if (mx_out_bf16) return gemm_launch_mxn_mx(p, d->block_m, d->grid_m, swiglu, st);
     return gemm_launch_mxn(p, d->block_m, d->grid_m, swiglu, st);
   }
   if (d->w_layout != TK_W_STRIDED) return fail(TK_ERR_INVALID, "tk_moe_gemm: bad w_layout %d", d->w_layout);

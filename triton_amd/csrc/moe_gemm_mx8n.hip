@@ -429,109 +429,6 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8n_kernel(const GemmParams p) 
   }  // rounds
 }
 
-// MX-quantised output of the persistent kernel below: `mx_out_epilogue` with the operands of rows and columns taken
-// from LDS (bias_s by tile column, gam_s / dst_s by tile row, fetched a unit ahead) and with no branch around a store:
-// rows without a destination, columns past the end and the lanes that do not write a block's scale byte store to an
-// offset beyond the range of their buffer resource, which the hardware drops.
-template <int MFW, int NFW, bool SWIGLU>
-__device__ __forceinline__ void staged_mx_epilogue(const GemmParams& p, f32x16_t (&acc)[NFW][MFW], __amdgpu_buffer_rsrc_t yrsrc,
-                                                   __amdgpu_buffer_rsrc_t ysrsrc, const float* bias_s, const float* gam_s, const int* dst_s,
-                                                   int ncol_tile, int ncol0, int lr, int h) {
-  const int NOUT = SWIGLU ? p.N / 2 : p.N;
-  const float nalpha_log2e = -p.alpha * 1.4426950408889634f;
-  const float limit = p.has_limit ? p.limit : INFINITY;
-  constexpr int VO = SWIGLU ? 4 : 8;
-  constexpr int NB = SWIGLU ? 1 : NFW;
-  // every LDS operand up front: one round trip for the unit
-  f32x4_t bh[NFW][2][2];
-  float gh[MFW];
-  int dh[MFW];
-#pragma unroll
-  for (int f = 0; f < NFW; ++f)
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      bh[f][u][0] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 4 * h);
-      bh[f][u][1] = *reinterpret_cast<const f32x4_t*>(bias_s + ncol_tile + f * 32 + 16 * u + 8 + 4 * h);
-    }
-#pragma unroll
-  for (int j = 0; j < MFW; ++j) {
-    gh[j] = gam_s[j * 32 + lr];
-    dh[j] = dst_s[j * 32 + lr];
-  }
-#pragma unroll
-  for (int j = 0; j < MFW; ++j) {
-    const float g = gh[j];
-    const int dst = dh[j];
-    float o[NFW][2][VO];
-#pragma unroll
-    for (int f = 0; f < NFW; ++f)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(acc[f][j][8 * u + i] + bh[f][u][0][i]), f32_bits(acc[f][j][8 * u + 4 + i] + bh[f][u][1][i]), false, false);
-          v[i] = bits_f32(sw[0]);
-          v[4 + i] = bits_f32(sw[1]);
-        }
-#pragma unroll
-        for (int i = 0; i < VO; ++i) o[f][u][i] = SWIGLU ? swiglu_f(v[2 * i], v[2 * i + 1], nalpha_log2e, limit) * g : v[i] * g;
-      }
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      // block maximum of |o|: fmaxf returns its other operand for a NaN, so a NaN never wins and the block's scale comes
-      // from its finite values.  (N_out is a multiple of 32: a block lies below it whole or not at all, and one that does
-      // not is not stored.)
-      float m = 0.f;
-#pragma unroll
-      for (int f = 0; f < NFW; ++f) {
-        if (!SWIGLU && f != b) continue;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int i = 0; i < VO; ++i) m = __builtin_fmaxf(m, __builtin_fabsf(o[f][u][i]));
-      }
-      {
-        // the other lane half's maximum: after the swap the first register holds both halves' lanes 0..31, the second both
-        // halves' lanes 32..63
-        auto sw = __builtin_amdgcn_permlane32_swap(f32_bits(m), f32_bits(m), false, false);
-        m = __builtin_fmaxf(bits_f32(sw[0]), bits_f32(sw[1]));
-      }
-      const uint32_t sbits = mx_scale_bits(m, TK_E4M3, TK_MX_ROUND_UP);
-      const float inv = mx_inv_scale(sbits);
-      const int blk_col0 = SWIGLU ? ncol0 / 2 : ncol0 + b * 32;
-      const uint32_t soff = (dst >= 0 && h == 0 && blk_col0 < NOUT) ? (uint32_t)dst * (uint32_t)p.ys_stride_m + (uint32_t)(blk_col0 >> 5) : kDroppedStore;
-      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(sbits >> 23), ysrsrc, soff, 0, 0);
-#pragma unroll
-      for (int f = 0; f < NFW; ++f) {
-        if (!SWIGLU && f != b) continue;
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int col0 = SWIGLU ? (ncol0 + f * 32 + 16 * u + 8 * h) / 2 : ncol0 + f * 32 + 16 * u + 8 * h;
-          // No clamp to +-448 in front of the conversion: the scale is the smallest power of two >= max / 448 (the rounded
-          // quotient of an fp32 by 448 = 1.75 * 2^8 is a power of two only when the exact one is), scaling by a power of
-          // two is exact, so |o * inv| <= 448 for every finite block; with an infinite maximum inv is 0.
-          float qv[VO];
-#pragma unroll
-          for (int i = 0; i < VO; ++i) qv[i] = o[f][u][i] * inv;
-          const uint32_t off = (dst >= 0 && col0 < NOUT) ? (uint32_t)dst * (uint32_t)p.y_stride_m + (uint32_t)col0 : kDroppedStore;
-          int w0 = 0;
-          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[0], qv[1], w0, false);
-          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[2], qv[3], w0, true);
-          if constexpr (VO == 8) {
-            int w1 = 0;
-            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[4], qv[5], w1, false);
-            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(qv[6], qv[7], w1, true);
-            __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{(uint32_t)w0, (uint32_t)w1}, yrsrc, off, 0, 0);
-          } else {
-            __builtin_amdgcn_raw_buffer_store_b32((uint32_t)w0, yrsrc, off, 0, 0);
-          }
-        }
-      }
-    }
-  }
-}
-
 #ifdef TK_MX8_STAMPS
 // diagnostic build only: per workgroup, sums of shader-clock cycles spent in [0] the K loops' prologues, [1] the K
 // loops, [2] the preparation of the next unit, [3] the epilogues; [4] units, [5] K-stages, [6] whole kernel
@@ -775,9 +672,6 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
   };
 
   template_int<0> S0;
-  template_int<1> S1;
-  template_int<2> S2;
-  template_int<3> S3;
 
   auto stage = [&](auto nj_c, auto ws_c, int c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
@@ -852,7 +746,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
   int resolve_slot = -1;
   auto run = [&](auto nj_c) __attribute__((always_inline)) {
     constexpr int NJ = decltype(nj_c)::value;
-    const long long t_run = MX8_T();
+    [[maybe_unused]] const long long t_run = MX8_T();
     // the loads left in flight at the loop header are in the order the steady state leaves them in at the top of a
     // stage: activations, their scales, weights of stage 1, then of stage 2
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
@@ -884,7 +778,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
       read_xs(0, decltype(jc)::value, xs[0]);
     });
     __builtin_amdgcn_sched_barrier(0);
-    const long long t_loop = MX8_T();
+    [[maybe_unused]] const long long t_loop = MX8_T();
     MX8_ADD(0, t_loop - t_run);
     int c = 0;
     for (; c + UNR - 1 < nst; c += UNR)
@@ -896,7 +790,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
     MX8_ADD(5, nst);
   };
 
-  const long long t_kernel = MX8_T();
+  [[maybe_unused]] const long long t_kernel = MX8_T();
   if (pid >= 0) {
     Unit& cur = cur_unit;
     cur = tile_unit(pid);
@@ -924,7 +818,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
         if (nj == decltype(n_c)::value) run(n_c);
       });
       resolve_slot = -1;
-      const long long t_prep = MX8_T();
+      [[maybe_unused]] const long long t_prep = MX8_T();
 
       const int wcol = nw * NFW * FM;
       const int ncol0 = cur.pid_n * BN + wcol;
@@ -952,7 +846,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
         unit_pointers(nxt, up);
         first_loads();
       }
-      const long long t_epi = MX8_T();
+      [[maybe_unused]] const long long t_epi = MX8_T();
       MX8_ADD(2, t_epi - t_prep);
       if constexpr (MXOUT)
         staged_mx_epilogue<MFW, NFW, SWIGLU>(p, acc, yrsrc, ysrsrc, bias_s[up], gam_s[up], dst_s[up], wcol, ncol0, lr, h);

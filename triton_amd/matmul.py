@@ -320,10 +320,8 @@ def _matmul_mx_out(a, b, bias, a_ragged_metadata, gather_indx, scatter_indx, pre
         f"c_mx_scale must be [{y.shape[0]}, {n_out // MXFP_BLOCK_SIZE}], got {tuple(scale_data.shape)}"
     vals, scales = downcast_to_mxfp(y, out_dtype, axis=-1)
     scale_data.view(scales.shape).copy_(scales)
-    # (the reference records these on the caller's PrecisionConfig as well: triton_kernels/matmul.py:364-369,764-765)
-    precision_config.c_mx_scale = scale_out
-    precision_config.c_microblock_size = MXFP_BLOCK_SIZE
-    precision_config.c_value_pack_factor = 2 if fp4 else 1
+    # (the reference also records c_microblock_size / c_value_pack_factor on the caller's PrecisionConfig,
+    # triton_kernels/matmul.py:364-369; nothing here reads them back, and the caller's object is left as it was given)
     if c is not None:
         assert tuple(c.shape[-2:]) == tuple(vals.shape) and c.dtype == vals.dtype
         c.view(vals.shape).copy_(vals)
@@ -504,6 +502,19 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         mx_out_fused = (mx_act and epilogue.specs.name == FnName.QUANTIZE_MXFP8.name
                         and precision_config.out_dtype == torch.float8_e4m3fn and precision_config.c_mx_scale is not None
                         and precision_config.c_microblock_size in (None, MXFP_BLOCK_SIZE))
+        if not mx_act and not extras:
+            # bf16 activations x tiled MXFP4 weights: the prefill kernel quantises its fp32 accumulator to e4m3, e5m2 or
+            # packed e2m1 (matmul_details/_matmul.py:593-637); other weight layouts take the two-step path below
+            fp4_out = epilogue.specs.name == FnName.QUANTIZE_MXFP4.name
+            n_out = b.shape[-1] // fused_activation.specs.reduction_n
+            a_plain = a.storage.data if isinstance(a, Tensor) else a
+            mx_out_fused = (isinstance(b, Tensor) and isinstance(b.storage.layout, GFX950MXValueLayout) and a_plain.dtype == torch.bfloat16
+                            and a_plain.ndim == 2 and precision_config.c_mx_scale is not None
+                            and precision_config.c_microblock_size in (None, MXFP_BLOCK_SIZE)
+                            and precision_config.out_dtype in ((torch.uint8, ) if fp4_out else (torch.float8_e4m3fn, torch.float8_e5m2))
+                            and n_out % MXFP_BLOCK_SIZE == 0 and b_ragged_metadata is None
+                            and (a_ragged_metadata is None or a_ragged_metadata.n_slices <= 1024)
+                            and (c is None or (c.ndim == 2 and c.stride(0) % 8 == 0 and c.data_ptr() % 8 == 0)))
         if mx_out_fused and extras:
             raise NotImplementedError("betas / out_alpha / c_acc_in are not supported together with the fused MX-output epilogue")
         if not mx_out_fused:
@@ -585,6 +596,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     y_rows = scatter_indx.shape[0] if scatter_indx is not None else M
     out_shape = (y_rows, N // reduction_n)
     c_scale = None
+    fp4_out = mx_out_fused and epilogue.specs.name == FnName.QUANTIZE_MXFP4.name
     if mx_out_fused:
         c_scale = precision_config.c_mx_scale
         if isinstance(c_scale, Tensor):
@@ -595,9 +607,8 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
             raise NotImplementedError(f"MX-quantised output needs N_out % 32 == 0 (got {out_shape[1]})")
         assert c_scale.dtype == torch.uint8 and tuple(c_scale.shape[-2:]) == (y_rows, out_shape[1] // MXFP_BLOCK_SIZE) \
             and c_scale.stride(-1) == 1, f"c_mx_scale must be uint8 [{y_rows}, {out_shape[1] // MXFP_BLOCK_SIZE}]"
-        # (recorded on the caller's PrecisionConfig, as the reference does: triton_kernels/matmul.py:364-369)
-        precision_config.c_microblock_size = MXFP_BLOCK_SIZE
-        precision_config.c_value_pack_factor = 1
+        if fp4_out:
+            out_shape = (y_rows, out_shape[1] // 2)  # two e2m1 codes per byte
     caller_c = c is not None
     if c is None:
         c = torch.empty(out_shape, dtype=out_dtype, device=a.device)
@@ -723,6 +734,10 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         from .matmul_details.opt_flags import _get_opt_flags_constraints
         forced = _get_opt_flags_constraints().get("block_m")
         block_m = 256 if (forced == 256 or (forced is None and is_ragged and M <= 144 * n_slices)) else 128
+    elif tiled and mx_out_fused:
+        from .matmul_details.opt_flags import _get_opt_flags_constraints
+        forced = _get_opt_flags_constraints().get("block_m")
+        block_m = 256 if (forced == 256 or (forced is None and is_ragged and M <= 144 * n_slices)) else 128  # the tile shapes with an MX-output epilogue
     elif tiled and extras:
         block_m = min(block_m, 32)  # the decode kernel carries the shared epilogue; the prefill kernels do not take these options
     elif tiled:
@@ -747,7 +762,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
     d.block_m = block_m
     d.M, d.N, d.K = M, N, K
     y_buf = c
-    if tiled and block_m >= 64 and not mx_act:
+    if tiled and block_m >= 64 and not mx_act and not mx_out_fused:
         # the prefill kernels write whole 16-byte pieces through a buffer resource: rows 16-byte aligned and padded to
         # a multiple of 8 columns; an output that is not goes through a padded buffer and is copied.  So does a
         # caller's own `c` whose last piece would spill past its columns (they may belong to a wider tensor).
@@ -755,7 +770,7 @@ def matmul(a, b, bias, a_ragged_metadata: RaggedTensorMetadata | None = None,
         if c.stride(0) % 8 or c.data_ptr() % 16 or c.stride(0) < n_pad or (caller_c and out_shape[1] % 8):
             y_buf = torch.empty((out_shape[0], n_pad), dtype=c.dtype, device=c.device)[:, :out_shape[1]]
     d.y = y_buf.data_ptr()
-    d.y_dtype = nt.TORCH_TO_TK[c.dtype]
+    d.y_dtype = nt.TK_E2M1 if fp4_out else nt.TORCH_TO_TK[c.dtype]
     d.y_stride_m = y_buf.stride(0)
     d.activation = act
     d.act_alpha, d.act_limit, d.act_has_limit = alpha, limit, has_limit
