@@ -167,6 +167,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   int32_t(*mask_s)[kDecMaskWords] = reinterpret_cast<int32_t(*)[kDecMaskWords]>(&red_s[0][0][0][0]);  // [expert][token word]: bit t = token t chose the expert
   for (int i = tid; i < E * kDecMaskWords; i += NT) (&mask_s[0][0])[i] = 0;
   __syncthreads();
+  DEC_STAMP(17);
   {
     const int l16 = lane & 15, sub = lane >> 4;
     for (int row0 = 0; row0 < T; row0 += NW * 4) {
@@ -186,6 +187,8 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
         key[i] = ordered_key(f);
         ret |= (e >= E ? 1u : 0u) << i;
       }
+      if (row0 == 0 && key[0] == 0x12345u) DEC_STAMP(9);  // (never true: makes the stamp below wait for the logits)
+      if (row0 == 0) DEC_STAMP(18);
       uint32_t sel_key[2] = {0u, 0u};
       int sel_idx[2] = {0, 0};
       uint32_t key0 = 0;
@@ -206,6 +209,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
           sel_idx[j >> 4] = idx;
         }
       }
+      if (row0 == 0) DEC_STAMP(19);
       // softmax over the k kept logits (fp32): z = exp(v - max) / sum
       float outv[2], z[2];
       const float vmax = key_to_float(key0);
@@ -314,6 +318,14 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   share(L0, L1, wg + 1, c0e, c1e);
   share(L2, L3, wg, c2b, c3b);
   share(L2, L3, wg + 1, c2e, c3e);
+  // A unit of either GEMM costs the same (one fragment's K-stages), and with a dozen units per workgroup one more in
+  // BOTH GEMMs is a sixth more work: the last run makes up for all the runs before it, so that a workgroup's units of the
+  // whole layer differ by at most one from any other's.  (With three units of that run per workgroup the cuts below grow
+  // with the workgroup index: its increment is at least L3 / G - 3.)
+  if (L3 >= 3 * (int64_t)G) {
+    c3b = wg * (U1 + U2) / G - (c0b + c1b) - c2b;
+    c3e = (wg + 1) * (U1 + U2) / G - (c0e + c1e) - c2e;
+  }
   const int64_t r0b = c0b, r0e = c0e, r1b = L0 + c1b, r1e = L0 + c1e;
   const int64_t r2b = c2b, r2e = c2e, r3b = L2 + c3b, r3e = L2 + c3e;
   int nr0 = (int)(r0e - r0b), nr1 = (int)(r1e - r1b), nr2 = (int)(r2e - r2b), nr3 = (int)(r3e - r3b);
@@ -409,7 +421,38 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       }
     }
   };
+  // this wave's K-slice of the x rows of a GEMM-1 unit's row block (tokens through the expert-sorted order)
+  auto fetch_x1 = [&](const DecUnit& u) __attribute__((always_inline)) {
+    const int a = (u.key >> 8) & 0xFFFF, rb = u.key & 0xFF;
+    const int e = act_s[a];
+    const int cnt = hist_s[e];
+    const int row0 = offs_s[e] + rb * 16;
+    const int rows = cnt - rb * 16 < 16 ? cnt - rb * 16 : 16;
+    const int row = lr < rows ? lr : rows - 1;
+    // first k of this lane in its wave's slice (opaque: otherwise the twelve addresses below are computed once, ahead
+    // of the loop, and parked in scratch memory, which turns every reload into a chain of dependent memory round trips)
+    int kb = wave * (XS * 128) + kg * 32;
+    asm volatile("" : "+v"(kb));
+    const int token = rowflat_s[row0 + row] / k;
+    const uint32_t base = (uint32_t)token * (uint32_t)(p.x_stride * 2);
+#pragma unroll
+    for (int j = 0; j < XS; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        int k0 = kb + j * 128 + t * 8;
+        k0 = k0 < p.K1 - 8 ? k0 : p.K1 - 8;  // past K the weights are zero (padding) or their scales are zeroed (stages past the last)
+        xr[j][t] = *reinterpret_cast<const u32x4_t*>(p.x + (base + (uint32_t)k0 * 2u));
+      }
+  };
+  int cur_key = 0;
   if (n_units > 0) {
+    // the first unit's activation slice is requested in front of the weight blocks (a wave's requests are answered in
+    // order, and the three units of weight blocks primed below keep the memory system busy for microseconds)
+    const DecUnit first = uniform_unit(0);
+    if ((first.key >> 24) == 1) {
+      fetch_x1(first);
+      cur_key = first.key;
+    }
     static_for<0, RD>([&](auto h_c) __attribute__((always_inline)) {
       const DecUnit u = uniform_unit(decltype(h_c)::value);
 #pragma unroll
@@ -457,7 +500,6 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   DEC_STAMP(12);
   bias_fetch(0);
   DEC_STAMP(13);
-  int cur_key = 0;
   // A finished GEMM-1 run is counted in without draining the wave's memory queue.  A wave's loads and stores complete
   // in issue order.  The epilogue of a run's last unit stores its rows of h right behind that unit's barrier; the
   // next unit opens another row block (or the other GEMM), so EVERY wave starts it by fetching new activation rows
@@ -520,16 +562,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
             xr[j][t] = __builtin_amdgcn_raw_buffer_load_b128(hrsrc, base + (uint32_t)k0 * 2u, 0, kThrough);
           }
       } else {
-        const int token = rowflat_s[row0 + row] / k;
-        const uint32_t base = (uint32_t)token * (uint32_t)(p.x_stride * 2);
-#pragma unroll
-        for (int j = 0; j < XS; ++j)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            int k0 = kb + j * 128 + t * 8;
-            k0 = k0 < K - 8 ? k0 : K - 8;
-            xr[j][t] = *reinterpret_cast<const u32x4_t*>(p.x + (base + (uint32_t)k0 * 2u));
-          }
+        fetch_x1(cur);
       }
     }
     if (i == 0) DEC_STAMP(14);
