@@ -438,6 +438,46 @@ def test_matmul_fp8(mods, device, m, n, k, layout, block_m, do_gather, do_scatte
     assert_allclose_gate(ref, y, what="fp8 y")
 
 
+@pytest.mark.parametrize("do_gather, do_scatter", [(True, False), (False, True)])
+def test_matmul_fp8_long_k_takes_the_wide_tiles(mods, device, monkeypatch, do_gather, do_scatter):
+    """With at least 512 rows per slice and K >= 8192 `matmul` picks row blocks of 256 for tiled e4m3 weights (256 x 256
+    tiles, every row fragment multiplied): two slices of 700 and 900 rows (partly filled last blocks), K = 8192, against
+    the oracle; the descriptor is checked to ask for block_m 256."""
+    mm, _, tensor = mods
+    from triton_amd import _native as nt
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import make_default_matmul_fp8_w_layout
+    g = torch.Generator().manual_seed(97)
+    m, n, k, n_slices = 1600, 320, 8192, 2
+    xq, sx, wq, sw = _fp8_operands(m, n, k, n_slices, g)
+    bias = torch.randn((n_slices, n), generator=g)
+    sizes = torch.tensor([700, 900], dtype=torch.int32)
+    md = tensor.make_ragged_tensor_metadata(sizes.to(device), m)
+    gi = torch.randint(0, m, (m, ), generator=g).to(torch.int32) if do_gather else None
+    sc = torch.randperm(m, generator=g).to(torch.int32) if do_scatter else None
+    wd = convert_layout(wrap_torch_tensor(wq.to(device).transpose(-1, -2).contiguous().transpose(-1, -2)), make_default_matmul_fp8_w_layout())
+    pc = mm.PrecisionConfig(a_mx_tensor_scale=sx.to(device), b_mx_tensor_scale=sw.to(device), out_dtype=torch.bfloat16)
+    seen = []
+    real_lib = nt.lib()
+
+    class Spy:
+        def tk_moe_gemm(self, d, stream):
+            seen.append(int(d.block_m))
+            return real_lib.tk_moe_gemm(d, stream)
+
+        def __getattr__(self, name):
+            return getattr(real_lib, name)
+
+    spy = Spy()
+    monkeypatch.setattr(mm.nt, "lib", lambda: spy)
+    dv = lambda t: None if t is None else t.to(device)
+    y = mm.matmul(xq.to(device), wd, bias.to(device), md, gather_indx=dv(gi), scatter_indx=dv(sc), precision_config=pc)
+    assert seen == [256], f"block_m asked of tk_moe_gemm: {seen}"
+    ref = omoe.matmul(xq, wq, bias, sizes, gather_indx=gi, scatter_indx=sc, x_row_scale=sx, w_col_scale=sw)
+    assert_close(ref, y, maxtol=2e-2, what="fp8 y, 256-row tiles")
+    assert_allclose_gate(ref, y, what="fp8 y, 256-row tiles")
+
+
 @pytest.mark.parametrize("per_expert", [False, True])
 def test_flexpoint_input_scales(mods, device, per_expert):
     """`FlexCtx(lhs_data=InFlexData(scale=...), rhs_data=InFlexData(scale=...))`: fp8 operands with one-element device

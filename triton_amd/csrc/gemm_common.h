@@ -78,6 +78,7 @@ int32_t gemm_launch_mxn(const GemmParams& p, int block_m, int grid_m, bool swigl
 int32_t gemm_launch_mxn_mx(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);  // block_m 128 / 256, MX-quantised output
 int32_t gemm_launch_mxd(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
 int32_t gemm_launch_f8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, hipStream_t st);
+int32_t gemm_launch_f8w(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st);  // 256 x 256 tiles (row blocks of 256)
 int32_t gemm_launch_mx8n(const GemmParams& p, int block_m, int grid_m, bool swiglu, bool mx_out, hipStream_t st);
 
 // Slices (experts) whose row and block offsets the persistent MXFP4 prefill kernel keeps in LDS: a tile's coordinates

@@ -121,6 +121,11 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
     if (d->n_slices > 1 && d->w_stride_e < nfr * nst * 8192) return fail(TK_ERR_INVALID, "tk_moe_gemm: expert stride smaller than one tiled expert");
     p.w_stride_e = d->w_stride_e;
     p.w_nst = (int32_t)nst;
+    if (d->block_m == 256) {
+      // 256 x 256 tiles; the kernel addresses activation rows with 32-bit byte offsets from x
+      const int64_t x_rows = d->x_rows > 0 ? d->x_rows : (d->gather_indx ? 0 : d->M);
+      if (x_rows > 0 && d->x_stride_m >= 0 && x_rows * d->x_stride_m < ((int64_t)1 << 32)) return gemm_launch_f8w(p, d->grid_m, swiglu, st);
+    }
     return gemm_launch_f8n(p, d->block_m, d->grid_m, swiglu, st);
   }
   if (mx_act) {
