@@ -795,27 +795,51 @@ __device__ __forceinline__ void fused_prefill_combine(const GemmParams& p, int t
   const __amdgpu_buffer_rsrc_t ysrc = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, p.y_bytes, 0x00020000);
   const uint32_t row_bytes = (uint32_t)(p.y_stride_m * 2);
   constexpr int kAround = 1 | 16;  // sc0 | sc1
-  for (int t = blockIdx.x; t < T; t += grid) {
-    for (int c = tid; c < n8; c += NT) {
-      float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (int j0 = 0; j0 < k; j0 += 4) {
-        u32x4_t v[4];
+  // The tokens of this workgroup and their 8-column groups form one index space, H items of it per lane and pass:
+  // their rows are all requested before any is summed (4 * H 16-byte loads in flight per lane when k <= 4).
+  constexpr int H = 2;
+  const int n_tok = blockIdx.x < T ? (T - 1 - blockIdx.x) / grid + 1 : 0;
+  const int items = n_tok * n8;
+  for (int i0 = tid; i0 < items; i0 += H * NT) {
+    int tt[H], cc[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const int i = i0 + h * NT;
+      const int lt = i / n8;
+      tt[h] = i < items ? blockIdx.x + lt * grid : -1;
+      cc[h] = i - lt * n8;
+    }
+    float sum[H][8];
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum[h][e] = 0.f;
+    for (int j0 = 0; j0 < k; j0 += 4) {
+      u32x4_t v[H][4];
+#pragma unroll
+      for (int h = 0; h < H; ++h)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t off = j0 + q < k ? (uint32_t)(t * k + j0 + q) * row_bytes + (uint32_t)c * 16u : kDroppedStore;
-          v[q] = __builtin_amdgcn_raw_buffer_load_b128(ysrc, off, 0, kAround);  // (dropped offsets read zero)
+          const uint32_t off =
+              (tt[h] >= 0 && j0 + q < k) ? (uint32_t)(tt[h] * k + j0 + q) * row_bytes + (uint32_t)cc[h] * 16u : kDroppedStore;
+          v[h][q] = __builtin_amdgcn_raw_buffer_load_b128(ysrc, off, 0, kAround);  // (dropped offsets read zero)
         }
+#pragma unroll
+      for (int h = 0; h < H; ++h)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            sum[2 * e] += bits_f32(v[q][e] << 16);
-            sum[2 * e + 1] += bits_f32(v[q][e] & 0xFFFF0000u);
+            sum[h][2 * e] += bits_f32(v[h][q][e] << 16);
+            sum[h][2 * e + 1] += bits_f32(v[h][q][e] & 0xFFFF0000u);
           }
-      }
-      *reinterpret_cast<u32x4_t*>(p.combine_out + (int64_t)t * p.combine_stride + c * 8) =
-          u32x4_t{pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3]), pack_bf16x2(sum[4], sum[5]), pack_bf16x2(sum[6], sum[7])};
     }
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+      if (tt[h] >= 0)
+        *reinterpret_cast<u32x4_t*>(p.combine_out + (int64_t)tt[h] * p.combine_stride + cc[h] * 8) =
+            u32x4_t{pack_bf16x2(sum[h][0], sum[h][1]), pack_bf16x2(sum[h][2], sum[h][3]), pack_bf16x2(sum[h][4], sum[h][5]),
+                    pack_bf16x2(sum[h][6], sum[h][7])};
   }
   __syncthreads();
   if (tid == 0) {
