@@ -165,13 +165,11 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   // with a minimum): ties go to the lower expert, as the reference's packed sort key does
   // (topk_details/_topk_forward.py:27-35,61).  No lane leaves its row, so the four tokens cost what one costs.
   int32_t(*mask_s)[kDecMaskWords] = reinterpret_cast<int32_t(*)[kDecMaskWords]>(&red_s[0][0][0][0]);  // [expert][token word]: bit t = token t chose the expert
-  for (int i = tid; i < E * kDecMaskWords; i += NT) (&mask_s[0][0])[i] = 0;
-  __syncthreads();
-  DEC_STAMP(17);
   {
     const int l16 = lane & 15, sub = lane >> 4;
     for (int row0 = 0; row0 < T; row0 += NW * 4) {
-      if (row0 + wave * 4 >= T) break;  // (a wave without tokens stays out of the others' way)
+      const bool wave_has_rows = row0 + wave * 4 < T;  // (uniform) a wave without tokens stays out of the others' way
+      if (!wave_has_rows && row0 > 0) break;
       const int row = row0 + wave * 4 + sub;
       const bool row_ok = row < T;
       uint32_t key[VPL];
@@ -187,6 +185,12 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
         key[i] = ordered_key(f);
         ret |= (e >= E ? 1u : 0u) << i;
       }
+      if (row0 == 0) {  // the masks are cleared while the first logits are on their way (every wave comes through here)
+        for (int i = tid; i < E * kDecMaskWords; i += NT) (&mask_s[0][0])[i] = 0;
+        __syncthreads();
+        DEC_STAMP(17);
+      }
+      if (!wave_has_rows) break;
       if (row0 == 0 && key[0] == 0x12345u) DEC_STAMP(9);  // (never true: makes the stamp below wait for the logits)
       if (row0 == 0) DEC_STAMP(18);
       uint32_t sel_key[2] = {0u, 0u};
@@ -301,19 +305,22 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   // When a workgroup reaches a GEMM-2 run, the rows of h it needs were finished (by all workgroups) a whole run
   // earlier, so the hand-over between the GEMMs costs no waiting.
   const int bh = (nblk + 1) >> 1;  // row blocks of the first half
-  const int64_t U1 = (int64_t)nblk * p.nfr1, U2 = (int64_t)nblk * p.nfr2;
-  const int64_t L0 = (int64_t)bh * p.nfr1, L1 = U1 - L0, L2 = (int64_t)bh * p.nfr2, L3 = U2 - L2;
-  const int64_t wg = blockIdx.x;
+  // (32-bit arithmetic: nblk <= 272 and nfr1 + nfr2 <= 288, so G * (U1 + U2) stays below 2^25; a 64-bit division is
+  // a hundred instructions, and a dozen of them stood between the routing and the first weight request)
+  const int U1 = nblk * p.nfr1, U2 = nblk * p.nfr2;
+  const int L0 = bh * p.nfr1, L1 = U1 - L0, L2 = bh * p.nfr2, L3 = U2 - L2;
+  const int wg = blockIdx.x;
+  auto udiv = [](int a, int b) -> int { return (int)((uint32_t)a / (uint32_t)b); };
   // Shares: the first run of each GEMM is cut evenly; the second makes up for it, so that a workgroup's units of
   // ONE GEMM differ by at most one from any other's (the GEMM-2 runs wait for everybody's GEMM-1 runs: what counts is
   // when the slowest workgroup finishes a GEMM).
-  auto share = [&](int64_t La, int64_t Lb, int64_t i, int64_t& a_cut, int64_t& b_cut) {
-    a_cut = i * La / G;
+  auto share = [&](int La, int Lb, int i, int& a_cut, int& b_cut) {
+    a_cut = udiv(i * La, G);
     // (with at least two units of the second run per workgroup the difference below grows with i; otherwise the
     // second run is cut evenly as well)
-    b_cut = Lb >= 2 * (int64_t)G ? i * (La + Lb) / G - a_cut : i * Lb / G;
+    b_cut = Lb >= 2 * G ? udiv(i * (La + Lb), G) - a_cut : udiv(i * Lb, G);
   };
-  int64_t c0b, c1b, c0e, c1e, c2b, c3b, c2e, c3e;
+  int c0b, c1b, c0e, c1e, c2b, c3b, c2e, c3e;
   share(L0, L1, wg, c0b, c1b);
   share(L0, L1, wg + 1, c0e, c1e);
   share(L2, L3, wg, c2b, c3b);
@@ -322,13 +329,13 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   // BOTH GEMMs is a sixth more work: the last run makes up for all the runs before it, so that a workgroup's units of the
   // whole layer differ by at most one from any other's.  (With three units of that run per workgroup the cuts below grow
   // with the workgroup index: its increment is at least L3 / G - 3.)
-  if (L3 >= 3 * (int64_t)G) {
-    c3b = wg * (U1 + U2) / G - (c0b + c1b) - c2b;
-    c3e = (wg + 1) * (U1 + U2) / G - (c0e + c1e) - c2e;
+  if (L3 >= 3 * G) {
+    c3b = udiv(wg * (U1 + U2), G) - (c0b + c1b) - c2b;
+    c3e = udiv((wg + 1) * (U1 + U2), G) - (c0e + c1e) - c2e;
   }
-  const int64_t r0b = c0b, r0e = c0e, r1b = L0 + c1b, r1e = L0 + c1e;
-  const int64_t r2b = c2b, r2e = c2e, r3b = L2 + c3b, r3e = L2 + c3e;
-  int nr0 = (int)(r0e - r0b), nr1 = (int)(r1e - r1b), nr2 = (int)(r2e - r2b), nr3 = (int)(r3e - r3b);
+  const int r0b = c0b, r0e = c0e, r1b = L0 + c1b, r1e = L0 + c1e;
+  const int r2b = c2b, r2e = c2e, r3b = L2 + c3b, r3e = L2 + c3e;
+  int nr0 = r0e - r0b, nr1 = r1e - r1b, nr2 = r2e - r2b, nr3 = r3e - r3b;
   if (nr0 + nr1 + nr2 + nr3 > kDecMaxUnits) {  // (the host's bound rules this out)
     if (tid == 0) atomicOr(&p.sync[1], 2);
     nr0 = nr0 < kDecMaxUnits ? nr0 : kDecMaxUnits;
@@ -348,10 +355,10 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       u.frag = 0;
     } else {
       const bool ph2 = i >= n1;
-      const int64_t uu = i < nr0 ? r0b + i : i < n1 ? r1b + (i - nr0) : i < n1 + nr2 ? r2b + (i - n1) : r3b + (i - n1 - nr2);
+      const int uu = i < nr0 ? r0b + i : i < n1 ? r1b + (i - nr0) : i < n1 + nr2 ? r2b + (i - n1) : r3b + (i - n1 - nr2);
       const int nfr = ph2 ? p.nfr2 : p.nfr1;
       const int nst = ph2 ? p.nst2 : p.nst1;
-      const int B = (int)(uu / nfr), F = (int)(uu - (int64_t)B * nfr);
+      const int B = udiv(uu, nfr), F = uu - B * nfr;
       int lo = 0, hi = A;  // last a with bpre[a] <= B
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -411,13 +418,13 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
     return u;
   };
   // counts GEMM-1 units [from, to) of this workgroup in at their row blocks' counters (unit u belongs to block u / nfr1)
-  auto signal_blocks = [&](int64_t ub, int64_t ue) __attribute__((always_inline)) {
+  auto signal_blocks = [&](int ub, int ue) __attribute__((always_inline)) {
     if (ue > ub) {
-      const int b_first = (int)(ub / p.nfr1), b_last = (int)((ue - 1) / p.nfr1);
+      const int b_first = udiv(ub, p.nfr1), b_last = udiv(ue - 1, p.nfr1);
       for (int b = b_first + tid; b <= b_last; b += NT) {
-        const int64_t lo = (int64_t)b * p.nfr1, hi = lo + p.nfr1;
-        const int64_t from = lo > ub ? lo : ub, to = hi < ue ? hi : ue;
-        __hip_atomic_fetch_add(&p.sync[2 + b * kDecBlockStride], (int)(to - from), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int lo = b * p.nfr1, hi = lo + p.nfr1;
+        const int from = lo > ub ? lo : ub, to = hi < ue ? hi : ue;
+        __hip_atomic_fetch_add(&p.sync[2 + b * kDecBlockStride], to - from, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   };
