@@ -311,28 +311,25 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   const int L0 = bh * p.nfr1, L1 = U1 - L0, L2 = bh * p.nfr2, L3 = U2 - L2;
   const int wg = blockIdx.x;
   auto udiv = [](int a, int b) -> int { return (int)((uint32_t)a / (uint32_t)b); };
-  // Shares: the first run of each GEMM is cut evenly; the second makes up for it, so that a workgroup's units of
-  // ONE GEMM differ by at most one from any other's (the GEMM-2 runs wait for everybody's GEMM-1 runs: what counts is
-  // when the slowest workgroup finishes a GEMM).
-  auto share = [&](int La, int Lb, int i, int& a_cut, int& b_cut) {
-    a_cut = udiv(i * La, G);
-    // (with at least two units of the second run per workgroup the difference below grows with i; otherwise the
-    // second run is cut evenly as well)
-    b_cut = Lb >= 2 * G ? udiv(i * (La + Lb), G) - a_cut : udiv(i * Lb, G);
+  // Shares.  The four runs are cut as one list: cut i of a run = floor(i * (S + L) / G) - floor(i * S / G), S = the
+  // units of the runs in front of it, L its own, so that what a workgroup has got from the runs so far is
+  // floor((i + 1) * S / G) - floor(i * S / G) whatever the remainders were: a workgroup's units of the whole layer
+  // differ by at most one from any other's, and so do its units of GEMM 1 (the GEMM-2 runs wait for everybody's
+  // GEMM-1 runs).  A unit of either GEMM costs the same, and with a dozen units per workgroup one more in every run is a
+  // quarter more work.  The cuts grow with i when L >= 2 G (their increment is at least L / G - 2); a shorter run is cut
+  // evenly by itself and the list starts again with it.
+  int S = 0;
+  auto share = [&](int L, int& cut_b, int& cut_e) {
+    if (S != 0 && L < 2 * G) S = 0;
+    cut_b = udiv(wg * (S + L), G) - udiv(wg * S, G);
+    cut_e = udiv((wg + 1) * (S + L), G) - udiv((wg + 1) * S, G);
+    S += L;
   };
   int c0b, c1b, c0e, c1e, c2b, c3b, c2e, c3e;
-  share(L0, L1, wg, c0b, c1b);
-  share(L0, L1, wg + 1, c0e, c1e);
-  share(L2, L3, wg, c2b, c3b);
-  share(L2, L3, wg + 1, c2e, c3e);
-  // A unit of either GEMM costs the same (one fragment's K-stages), and with a dozen units per workgroup one more in
-  // BOTH GEMMs is a sixth more work: the last run makes up for all the runs before it, so that a workgroup's units of the
-  // whole layer differ by at most one from any other's.  (With three units of that run per workgroup the cuts below grow
-  // with the workgroup index: its increment is at least L3 / G - 3.)
-  if (L3 >= 3 * G) {
-    c3b = udiv(wg * (U1 + U2), G) - (c0b + c1b) - c2b;
-    c3e = udiv((wg + 1) * (U1 + U2), G) - (c0e + c1e) - c2e;
-  }
+  share(L0, c0b, c0e);
+  share(L1, c1b, c1e);
+  share(L2, c2b, c2e);
+  share(L3, c3b, c3e);
   const int r0b = c0b, r0e = c0e, r1b = L0 + c1b, r1e = L0 + c1e;
   const int r2b = c2b, r2e = c2e, r3b = L2 + c3b, r3e = L2 + c3e;
   int nr0 = r0e - r0b, nr1 = r1e - r1b, nr2 = r2e - r2b, nr3 = r3e - r3b;
