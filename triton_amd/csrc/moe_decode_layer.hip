@@ -43,6 +43,7 @@ constexpr int kDecBlockWords = (kDecMaxRows + kDecMaxRows / 16) * kDecBlockStrid
 struct DecodeParams {
   const uint8_t* x;  // bf16 [T, K1]
   int64_t x_stride;  // elements
+  uint32_t x_bytes;  // extent of x (the rows are read through a buffer resource)
   const void* logits;
   int64_t logits_stride;
   int32_t logits_is_bf16;
@@ -149,6 +150,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   __shared__ DecUnit tab_s[kDecMaxUnits + kDecRing];
   __shared__ __attribute__((aligned(16))) float red_s[2][NW][64][8];
   __shared__ __attribute__((aligned(16))) float bias_s[kDecMaxUnits][32];  // bias of a unit's 32 columns
+  __shared__ u32x4_t xst_s[NW][4][64];  // per wave: one K-stage of a row block's activations on its way into MFMA order
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -393,8 +395,11 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
                                 // stay exact only in straight-line code); their scales are taken as zero when they are used
 #pragma unroll
     for (int g = 0; g < 2; ++g) {
-      wr[H][j][g] = *reinterpret_cast<const u32x4_t*>(u.w + (int64_t)s * 2048 + g * 256 + wlane);
-      sr[H][j][g] = *reinterpret_cast<const uint32_t*>(u.s + (int64_t)s * 128 + g * 64 + slane);
+      // (global address space spelled out: the pointers come out of the LDS table, the compiler takes them for generic
+      // ones, and with FLAT loads in flight every wait for memory on this target is a wait for ALL of it, i.e. the ring
+      // of weight blocks would be drained at the head of every unit)
+      wr[H][j][g] = *(const __attribute__((address_space(1))) u32x4_t*)(u.w + (int64_t)s * 2048 + g * 256 + wlane);
+      sr[H][j][g] = *(const __attribute__((address_space(1))) uint32_t*)(u.s + (int64_t)s * 128 + g * 64 + slane);
     }
   };
   auto unit_nst = [&](const DecUnit& u) __attribute__((always_inline)) -> int { return (u.key >> 24) == 2 ? p.nst2 : p.nst1; };
@@ -425,36 +430,70 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       }
     }
   };
-  // this wave's K-slice of the x rows of a GEMM-1 unit's row block (tokens through the expert-sorted order)
-  auto fetch_x1 = [&](const DecUnit& u) __attribute__((always_inline)) {
+  // This wave's K-slice of a row block's activation rows: x through the expert-sorted order for GEMM 1, h for GEMM 2.
+  // The MFMA wants row lr's k-block kg in lane (lr, kg): loaded that way, the sixteen lanes that one pass of a load
+  // serves touch sixteen rows, i.e. sixteen cache lines for 16 bytes each.  So the rows are loaded four lanes to a row
+  // (lane = row * 4 + chunk: 64 contiguous bytes per row and instruction, rows past the block's last dropped, not
+  // repeated) and turned into MFMA order through a 4 KiB buffer of the wave's own in LDS, one K-stage at a time
+  // (LDS operations of a wave execute in order; 16-byte chunks swizzled by the row so that neither side conflicts).
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.x), 0, p.x_bytes, 0x00020000);
+  auto x_request = [&](auto ph_c, const DecUnit& u) __attribute__((always_inline)) {
+    constexpr int ph = decltype(ph_c)::value;  // 1: rows of x, 2: rows of h
     const int a = (u.key >> 8) & 0xFFFF, rb = u.key & 0xFF;
     const int e = act_s[a];
     const int cnt = hist_s[e];
     const int row0 = offs_s[e] + rb * 16;
     const int rows = cnt - rb * 16 < 16 ? cnt - rb * 16 : 16;
-    const int row = lr < rows ? lr : rows - 1;
+    const int r = lane >> 2, c = lane & 3;
+    const bool valid = r < rows;
+    const int K = ph == 2 ? p.K2 : p.K1;
     // first k of this lane in its wave's slice (opaque: otherwise the twelve addresses below are computed once, ahead
     // of the loop, and parked in scratch memory, which turns every reload into a chain of dependent memory round trips)
-    int kb = wave * (XS * 128) + kg * 32;
+    int kb = wave * (XS * 128) + c * 8;
     asm volatile("" : "+v"(kb));
-    const int token = rowflat_s[row0 + row] / k;
-    const uint32_t base = (uint32_t)token * (uint32_t)(p.x_stride * 2);
+    uint32_t base;
+    if constexpr (ph == 2) {
+      base = (uint32_t)(row0 + r) * (uint32_t)(p.K2 * 2);
+    } else {
+      const int token = rowflat_s[row0 + (valid ? r : 0)] / k;
+      base = (uint32_t)token * (uint32_t)(p.x_stride * 2);
+    }
 #pragma unroll
     for (int j = 0; j < XS; ++j)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        int k0 = kb + j * 128 + t * 8;
-        k0 = k0 < p.K1 - 8 ? k0 : p.K1 - 8;  // past K the weights are zero (padding) or their scales are zeroed (stages past the last)
-        xr[j][t] = *reinterpret_cast<const u32x4_t*>(p.x + (base + (uint32_t)k0 * 2u));
+      for (int q = 0; q < 4; ++q) {
+        const int k0 = kb + j * 128 + q * 32;
+        // past K the weights are zero (padding) or their scales are zeroed (stages past the last): zeros will do
+        const uint32_t off = (valid && k0 < K) ? base + (uint32_t)k0 * 2u : kDroppedStore;
+        if constexpr (ph == 2)
+          xr[j][q] = __builtin_amdgcn_raw_buffer_load_b128(hrsrc, off, 0, kThrough);
+        else
+          xr[j][q] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 0, 0);
       }
+  };
+  auto x_settle = [&]() __attribute__((always_inline)) {
+    const int r = lane >> 2, c = lane & 3;
+    const int wpos = r * 4 + (c ^ ((r >> 2) & 3));
+#pragma unroll
+    for (int j = 0; j < XS; ++j) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xst_s[wave][q][wpos] = xr[j][q];
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xr[j][t] = xst_s[wave][kg][lr * 4 + (t ^ ((lr >> 2) & 3))];
+    }
   };
   int cur_key = 0;
   if (n_units > 0) {
     // the first unit's activation slice is requested in front of the weight blocks (a wave's requests are answered in
     // order, and the three units of weight blocks primed below keep the memory system busy for microseconds)
     const DecUnit first = uniform_unit(0);
-    if ((first.key >> 24) == 1) {
-      fetch_x1(first);
+    const bool x_first = (first.key >> 24) == 1;
+    if (x_first) {
+      x_request(std::integral_constant<int, 1>{}, first);
       cur_key = first.key;
     }
     static_for<0, RD>([&](auto h_c) __attribute__((always_inline)) {
@@ -462,6 +501,9 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
       for (int j = 0; j < XS; ++j) load_w(h_c, j, u, unit_nst(u));
     });
+    // (here, in straight-line code behind the requests, the wait in front of the LDS writes counts the weight blocks
+    // out: behind the bias loops below it would be a wait for everything requested so far)
+    if (x_first) x_settle();
   }
   // The biases of this workgroup's units (32 columns each) go to LDS once: requested behind the first weight blocks,
   // written in front of the first unit's barrier.  Four values per thread cover 64 units; more take another round.
@@ -527,11 +569,6 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
     if (cur.key != cur_key) {
       cur_key = cur.key;
       // ---- a new (expert, row block): this wave's K-slice of its activation rows goes into registers ----
-      const int row = lr < rows ? lr : rows - 1;
-      // first k of this lane in its wave's slice (opaque: otherwise the twelve addresses below are computed once, ahead
-      // of the loop, and parked in scratch memory, which turns every reload into a chain of dependent memory round trips)
-      int kb = wave * (XS * 128) + kg * 32;
-      asm volatile("" : "+v"(kb));
       if (ph == 2) {
         const int blk = bpre_s[a] + rb;  // a block of the first half was computed by run 0 alone
         if (!signalled0 || (blk >= bh && !signalled)) {  // (uniform) see above: count in what this workgroup itself still owes
@@ -556,18 +593,11 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
         }
         __syncthreads();
         if (i == n1) DEC_STAMP(5);
-        const uint32_t base = (uint32_t)(row0 + row) * (uint32_t)(p.K2 * 2);
-#pragma unroll
-        for (int j = 0; j < XS; ++j)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            int k0 = kb + j * 128 + t * 8;
-            k0 = k0 < K - 8 ? k0 : K - 8;  // past K the weights are zero (padding) or their scales are zeroed (stages past the last)
-            xr[j][t] = __builtin_amdgcn_raw_buffer_load_b128(hrsrc, base + (uint32_t)k0 * 2u, 0, kThrough);
-          }
+        x_request(std::integral_constant<int, 2>{}, cur);
       } else {
-        fetch_x1(cur);
+        x_request(std::integral_constant<int, 1>{}, cur);
       }
+      x_settle();
     }
     if (i == 0) DEC_STAMP(14);
     const bool leader = (i % NW) == wave;
@@ -793,6 +823,11 @@ extern "C" int32_t tk_moe_decode_layer(const tk_decode_layer_desc* d, tk_stream_
   DecodeParams p;
   p.x = static_cast<const uint8_t*>(d->x);
   p.x_stride = d->x_stride_m;
+  {
+    const int64_t extent = ((int64_t)(T - 1) * d->x_stride_m + d->d_model) * 2;
+    if (d->x_stride_m < d->d_model || extent > 0x7FFFFFFFll) return fail(TK_ERR_UNSUPPORTED, "tk_moe_decode_layer: activation rows must not overlap and must lie within 2 GiB (row stride %lld)", (long long)d->x_stride_m);
+    p.x_bytes = (uint32_t)extent;
+  }
   p.logits = d->logits;
   p.logits_stride = d->logits_stride_m;
   p.logits_is_bf16 = d->logits_dtype == TK_BF16;
