@@ -685,11 +685,15 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       }
     }
   };
-  for (int i = 0; i < n_units; i += RD) {
-    static_for<0, RD>([&](auto h_c) __attribute__((always_inline)) {
-      if (i + decltype(h_c)::value < n_units) unit_body(h_c, i + decltype(h_c)::value);
-    });
-  }
+  // Whole rounds of RD units run without a test between the units: with one, the compiler has to allow for a round
+  // that skips its later units and comes back to the first, i.e. for weight blocks that nothing younger follows, and
+  // its waits then drain the wave's memory queue once per round.
+  int i_unit = 0;
+  for (; i_unit + RD <= n_units; i_unit += RD)
+    static_for<0, RD>([&](auto h_c) __attribute__((always_inline)) { unit_body(h_c, i_unit + decltype(h_c)::value); });
+  static_for<0, RD - 1>([&](auto h_c) __attribute__((always_inline)) {
+    if (i_unit + decltype(h_c)::value < n_units) unit_body(h_c, i_unit + decltype(h_c)::value);
+  });
   DEC_STAMP(6);
   // ---- 4./5. hand-over of whatever is still to be counted in, then the combine of this workgroup's rows of y ----
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
