@@ -84,8 +84,8 @@ struct DecUnit {
 #ifdef TK_DEC_STAMPS
 __device__ long long dec_stamps[1024][20];
 #define DEC_STAMP(n) do { if (threadIdx.x == 0) dec_stamps[blockIdx.x][n] = (long long)__builtin_amdgcn_s_memrealtime(); } while (0)
-// end of unit i's K loop in four workgroups (rows 512..515 of the table, 20 columns x 2 rows each)
-#define DEC_UNIT_STAMP(i) do { if (threadIdx.x == 0 && (blockIdx.x & 63) == 5 && (i) < 40) dec_stamps[512 + (blockIdx.x >> 6) * 2 + (i) / 20][(i) % 20] = (long long)__builtin_amdgcn_s_memrealtime(); } while (0)
+// end of unit i's K loop in every workgroup (rows 512 + 2 * workgroup of the table, 20 columns x 2 rows each)
+#define DEC_UNIT_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 256 && (i) < 40) dec_stamps[512 + blockIdx.x * 2 + (i) / 20][(i) % 20] = (long long)__builtin_amdgcn_s_memrealtime(); } while (0)
 #else
 #define DEC_UNIT_STAMP(i) do {} while (0)
 #define DEC_STAMP(n) do {} while (0)
