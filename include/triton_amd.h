@@ -427,8 +427,8 @@ int32_t tk_ragged_k_gemm(const tk_ragged_k_desc* desc, tk_stream_t stream);
 #define TK_DECODE_MAX_ROWS 256
 #define TK_DECODE_MAX_EXPERTS 512
 typedef struct tk_decode_layer_desc {
-  const void* x; /* bf16 [n_tokens, d_model], unit stride along d_model */
-  int64_t x_stride_m;
+  const void* x; /* bf16 [n_tokens, d_model], unit stride along d_model, 16-byte aligned */
+  int64_t x_stride_m; /* elements; >= d_model, a multiple of 8, all rows within 2 GiB of x */
   const void* logits; /* [n_tokens, n_experts], TK_F32 or TK_BF16 */
   int32_t logits_dtype;
   int64_t logits_stride_m;

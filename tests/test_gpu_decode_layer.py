@@ -217,3 +217,16 @@ def test_fallback_and_refusals(api, device, gptoss_weights):
     h = api.matmul_ogs(x, W["w1"], W["b1"], rdata, gather_indx=gather, precision_config=pc1, fused_activation=act)
     want = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=pc2, gammas=rdata.gate_scal)
     assert torch.equal(out, want)
+    # activations whose rows are not contiguous take the three calls as well (the single launch reads rows of x 16 bytes
+    # at a time through a buffer resource), and give what the contiguous copy gives
+    xt = torch.randn((2880, 16), device=device).to(torch.bfloat16).t()  # [16, 2880] with unit stride along the tokens
+    lg = torch.randn((16, 128), device=device)
+    assert api.md.one_launch_reason(xt, lg, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act) is not None
+    assert api.md.one_launch_reason(xt.contiguous(), lg, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act) is None
+    a = api.md.moe_mlp(xt, lg, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)
+    rdata, gather, scatter = api.routing(lg, 4)
+    h = api.matmul_ogs(xt.contiguous(), W["w1"], W["b1"], rdata, gather_indx=gather, precision_config=pc1, fused_activation=act)
+    b = api.matmul_ogs(h, W["w2"], W["b2"], rdata, scatter_indx=scatter, precision_config=pc2, gammas=rdata.gate_scal)
+    assert torch.equal(a, b)
+    one = api.md.moe_mlp(xt.contiguous(), lg, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)  # (one launch: other K-split)
+    torch.testing.assert_close(one.float(), b.float(), atol=3e-2, rtol=3e-2)

@@ -90,6 +90,10 @@ def one_launch_reason(x, logits, n_expts_act, w1, b1, w2, b2, pc1, pc2, act) -> 
         return "weight shapes do not form an FFN over these activations"
     if d_model > MAX_DIM or d_ff > MAX_DIM or d_model % 8 or d_ff % 8:
         return "d_model and d_ff must be multiples of 8 up to 3072"
+    # (the kernel reads the rows of x through a 32-bit buffer resource, 16 bytes at a time)
+    if T and (x.stride(1) != 1 or x.stride(0) < d_model or x.stride(0) % 8 or x.data_ptr() % 16
+              or ((T - 1) * x.stride(0) + d_model) * 2 > 0x7FFFFFFF):
+        return "activation rows must be contiguous, 16-byte aligned, non-overlapping and within 2 GiB"
     for b, n in ((b1, n1), (b2, n2)):
         if b is not None and not (b.ndim == 2 and b.shape == (E, n) and b.stride(-1) == 1 and b.dtype in (torch.float32, torch.bfloat16)):
             return "biases must be [experts, N] in fp32 or bf16"
