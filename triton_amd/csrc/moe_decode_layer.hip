@@ -166,7 +166,9 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   // running (in-lane maximum, then four DPP steps inside the row) and the LOWEST expert index holding it (same again
   // with a minimum): ties go to the lower expert, as the reference's packed sort key does
   // (topk_details/_topk_forward.py:27-35,61).  No lane leaves its row, so the four tokens cost what one costs.
-  int32_t(*mask_s)[kDecMaskWords] = reinterpret_cast<int32_t(*)[kDecMaskWords]>(&red_s[0][0][0][0]);  // [expert][token word]: bit t = token t chose the expert
+  // [token word][expert]: bit t of word w = token 32 w + t chose the expert.  (Experts along the rows: in the other order the
+  // lanes of the counting pass below, which own neighbouring experts, all met in one LDS bank.)
+  int32_t(*mask_s)[kDecMaxExperts] = reinterpret_cast<int32_t(*)[kDecMaxExperts]>(&red_s[0][0][0][0]);
   {
     const int l16 = lane & 15, sub = lane >> 4;
     for (int row0 = 0; row0 < T; row0 += NW * 4) {
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
         ret |= (e >= E ? 1u : 0u) << i;
       }
       if (row0 == 0) {  // the masks are cleared while the first logits are on their way (every wave comes through here)
-        for (int i = tid; i < E * kDecMaskWords; i += NT) (&mask_s[0][0])[i] = 0;
+        for (int i = tid; i < kDecMaxExperts * ((T + 31) >> 5); i += NT) (&mask_s[0][0])[i] = 0;
         __syncthreads();
         DEC_STAMP(17);
       }
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
           e = e < 0 ? 0 : (e < E ? e : E - 1);  // (k <= E: every round finds a column)
           eid_s[row * k + j] = (int16_t)e;
           gate_s[row * k + j] = outv[q];
-          atomicOr(&mask_s[e][row >> 5], 1 << (row & 31));
+          atomicOr(&mask_s[row >> 5][e], 1 << (row & 31));
           if (blockIdx.x == 0) {
             if (p.indx_out) p.indx_out[row * k + j] = (int16_t)e;
             if (p.vals_out) p.vals_out[row * k + j] = outv[q];
@@ -252,7 +254,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   // ---- rows per expert, expert offsets, the list of active experts and their row blocks (wave 0) ----------
   const int tw = (T + 31) >> 5;  // token words in use
   if (wave == 0) {
-    constexpr int PER = kDecMaxExperts / 64;
+    constexpr int PER = VPL * 16 / 64;  // experts per lane (the kernel's variant covers VPL * 16 experts)
     int cnt[PER];
     int rows = 0, blks = 0, acts = 0;
 #pragma unroll
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       const int e = lane * PER + i;
       int c = 0;
       if (e < E)
-        for (int w = 0; w < tw; ++w) c += __builtin_popcount((uint32_t)mask_s[e][w]);
+        for (int w = 0; w < tw; ++w) c += __builtin_popcount((uint32_t)mask_s[w][e]);
       cnt[i] = c;
       rows += c;
       blks += (c + 15) >> 4;
@@ -294,8 +296,8 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   for (int f = tid; f < R; f += NT) {
     const int e = eid_s[f], t = f / k;
     int rank = 0;
-    for (int w = 0; w < (t >> 5); ++w) rank += __builtin_popcount((uint32_t)mask_s[e][w]);
-    rank += __builtin_popcount((uint32_t)mask_s[e][t >> 5] & ((1u << (t & 31)) - 1u));
+    for (int w = 0; w < (t >> 5); ++w) rank += __builtin_popcount((uint32_t)mask_s[w][e]);
+    rank += __builtin_popcount((uint32_t)mask_s[t >> 5][e] & ((1u << (t & 31)) - 1u));
     rowflat_s[offs_s[e] + rank] = (int16_t)f;
   }
   const int A = misc_s[0];
