@@ -148,7 +148,9 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
   __shared__ int32_t bpre_s[kDecMaxExperts + 1];  // a -> 16-row blocks of the active experts before a
   __shared__ int32_t misc_s[4];                   // [0] number of active experts
   __shared__ DecUnit tab_s[kDecMaxUnits + kDecRing];
-  __shared__ __attribute__((aligned(16))) float red_s[2][NW][64][8];
+  // partial sums of a unit: [unit parity][wave][half][lane] (a lane's two quads 1 KiB apart: 16-byte accesses of
+  // neighbouring lanes are then contiguous, without bank conflicts)
+  __shared__ f32x4_t red_s[2][NW][2][64];
   __shared__ __attribute__((aligned(16))) float bias_s[kDecMaxUnits][32];  // bias of a unit's 32 columns
   __shared__ u32x4_t xst_s[NW][4][64];  // per wave: one K-stage of a row block's activations on its way into MFMA order
 
@@ -635,9 +637,8 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
     DEC_UNIT_STAMP(i);
     if (i == 0) bias_park(0);
     {
-      float* mine = &red_s[i & 1][wave][lane][0];
-      *reinterpret_cast<f32x4_t*>(mine) = acc[0];
-      *reinterpret_cast<f32x4_t*>(mine + 4) = acc[1];
+      red_s[i & 1][wave][0][lane] = acc[0];
+      red_s[i & 1][wave][1][lane] = acc[1];
     }
     __syncthreads();
     if (i == 0) DEC_STAMP(16);
@@ -658,9 +659,8 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int q = 0; q < NW; ++q) {
-        const float* part = &red_s[i & 1][q][lane][0];
-        s0 += *reinterpret_cast<const f32x4_t*>(part);
-        s1 += *reinterpret_cast<const f32x4_t*>(part + 4);
+        s0 += red_s[i & 1][q][0][lane];
+        s1 += red_s[i & 1][q][1][lane];
       }
       const bool row_ok = lr < rows;
       if (ph == 1) {
