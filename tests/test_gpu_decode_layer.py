@@ -230,3 +230,20 @@ def test_fallback_and_refusals(api, device, gptoss_weights):
     assert torch.equal(a, b)
     one = api.md.moe_mlp(xt.contiguous(), lg, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)  # (one launch: other K-split)
     torch.testing.assert_close(one.float(), b.float(), atol=3e-2, rtol=3e-2)
+
+
+def test_padded_activation_rows_give_what_contiguous_rows_give(api, device, gptoss_weights):
+    """Rows of x with a pitch (a slice of a wider buffer): the single launch reads them through the row stride."""
+    W = gptoss_weights["tiled"]
+    act = api.act(1.702, 7.0)
+    pc1, pc2 = api.PrecisionConfig(b_mx_scale=W["w1s"]), api.PrecisionConfig(b_mx_scale=W["w2s"])
+    g = torch.Generator().manual_seed(11)
+    wide = torch.randn((24, 2880 + 64), generator=g).to(torch.bfloat16).to(device)
+    x = wide[:, 8:8 + 2880]  # pitch 2944 elements, first element 16 bytes into the buffer
+    logits = torch.randn((24, 128), generator=g).to(device)
+    assert x.stride(0) == 2944 and api.md.one_launch_reason(x, logits, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act) is None
+    a = api.md.moe_decode_layer(x, logits, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)
+    b = api.md.moe_decode_layer(x.contiguous(), logits, 4, W["w1"], W["b1"], W["w2"], W["b2"], pc1, pc2, act)
+    torch.cuda.synchronize()
+    assert api.md.workspace_error_word(x, logits, 4, W["w1"]) == 0
+    assert torch.equal(a, b)
