@@ -133,6 +133,9 @@ def test_heavy_skew_many_row_blocks_on_one_expert(api, device, gptoss_weights):
     (33, 12, 4, 256, 3072, torch.bfloat16, 7.0),    # the largest d_ff (every K-slice of GEMM 2 in use), ragged row blocks
     (16, 130, 1, 384, 192, None, 7.0),              # E > 128 (the wide-router variant), top-1, no biases
     (64, 4, 4, 3072, 512, torch.bfloat16, 5.0),     # the largest d_model, every token on every expert (4 blocks each)
+    (256, 16, 1, 128, 64, None, None),              # 256 tokens: every word of the token masks in use, top-1
+    (32, 512, 8, 128, 128, torch.float32, 7.0),     # the most experts (the wide router, eight experts per lane), top-8
+    (100, 64, 2, 2880, 64, torch.bfloat16, None),   # 200 routed rows over four mask words, gpt-oss d_model, a thin FFN
 ])
 def test_odd_shapes(api, device, T, E, k, d_model, d_ff, bias_dtype, limit):
     from bench import to_matmul_layout
