@@ -235,12 +235,17 @@ __device__ __forceinline__ const int32_t* ragged_metadata(const int32_t* slice_s
     }
     __syncthreads();
     if (threadIdx.x < kQuantities) {
+      // (only the waves that hold slices of this trip: with 128 experts two of the sixteen, and every step of this walk
+      // is an LDS round trip)
+      const int left = E - base;
+      const int used = left >= kScanThreads ? kScanWaves : (left + 63) >> 6;
       int run = 0;
-      for (int w = 0; w < kScanWaves; ++w) {
+      for (int w = 0; w < used; ++w) {
         const int t = wave_tot[threadIdx.x][w];
         wave_tot[threadIdx.x][w] = run;
         run += t;
       }
+      for (int w = used; w < kScanWaves; ++w) wave_tot[threadIdx.x][w] = run;
       wave_tot[threadIdx.x][kScanWaves] = run;
     }
     __syncthreads();
@@ -274,23 +279,25 @@ __device__ __forceinline__ const int32_t* ragged_metadata(const int32_t* slice_s
   if (!want_ragged) return use_lds ? offs_s[0] : nullptr;
   __threadfence_block();
   __syncthreads();
-#pragma unroll
-  for (int b = 0; b < kNumBlockSizes; ++b) {
+  // (the slots of all block sizes in ONE loop: with a few hundred slots per size the five searches of a thread, seven
+  // dependent LDS reads each, run side by side in different threads instead of one after the other)
+  const int n_slots = kNumBlockSizes * r.max_n_blocks;
+  for (int slot = threadIdx.x; slot < n_slots; slot += kScanThreads) {
+    const int b = slot / r.max_n_blocks, i = slot - b * r.max_n_blocks;
     const int32_t* offs = use_lds ? offs_s[1 + b] : r.block_offs + b * r.block_offs_stride;
-    int32_t* sched = r.block_sched + b * r.block_sched_stride;
-    const int total = carry[1 + b];
-    for (int i = threadIdx.x; i < r.max_n_blocks; i += kScanThreads) {
-      int val = -1;
-      if (i < total) {
-        int lo = 0, hi = E;  // largest e with offs[e] <= i; empty slices share an offset, the last one wins
-        while (hi - lo > 1) {
-          const int mid = (lo + hi) >> 1;
-          if (offs[mid] <= i) lo = mid; else hi = mid;
-        }
-        val = ((i - offs[lo]) << 16) | lo;
+    int tot = 0;  // blocks of this size in all slices (every thread has carried the totals through the scan)
+#pragma unroll
+    for (int bb = 0; bb < kNumBlockSizes; ++bb) tot = bb == b ? carry[1 + bb] : tot;
+    int val = -1;
+    if (i < tot) {
+      int lo = 0, hi = E;  // largest e with offs[e] <= i; empty slices share an offset, the last one wins
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (offs[mid] <= i) lo = mid; else hi = mid;
       }
-      sched[i] = val;
+      val = ((i - offs[lo]) << 16) | lo;
     }
+    r.block_sched[b * r.block_sched_stride + i] = val;
   }
   return use_lds ? offs_s[0] : nullptr;
 }
@@ -571,7 +578,7 @@ struct SmallParams {
 
 template <int DT, int EPL, bool PROVIDED>
 __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallParams q) {
-  __shared__ int32_t eid_s[kSmallEntries];
+  __shared__ __attribute__((aligned(16))) int32_t eid_s[kSmallEntries];
   __shared__ uint32_t val_s[kSmallEntries];
   __shared__ int32_t hist_s[kMaxExperts];
   __shared__ uint32_t words_s[kScanWaves][EPL * 2];
@@ -678,8 +685,16 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
     const int e = eid_s[f];
     int pos = -1;
     if (e >= 0) {
+      // entries of the same expert in front of this one: four per 16-byte LDS read, the reads independent of one
+      // another (one entry per read and trip was a chain of LDS round trips as long as the batch)
       int rank = 0;
-      for (int g = 0; g < f; ++g) rank += eid_s[g] == e ? 1 : 0;
+      const int f4 = f & ~3;
+#pragma unroll 4
+      for (int g = 0; g < f4; g += 4) {
+        const int4 v = *reinterpret_cast<const int4*>(&eid_s[g]);
+        rank += (v.x == e ? 1 : 0) + (v.y == e ? 1 : 0) + (v.z == e ? 1 : 0) + (v.w == e ? 1 : 0);
+      }
+      for (int g = f4; g < f; ++g) rank += eid_s[g] == e ? 1 : 0;
       pos = offs[e] + rank;
       q.col_sorted[pos] = f;
       if (q.gather_out) q.gather_out[pos] = f / k;
