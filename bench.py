@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
 
-A "step" is one forward pass of the gpt-oss-120b-shaped MXFP4 MoE FFN (BASELINE config 3: 4096 tokens,
+A "step" is one forward pass of the gpt-oss-120b-shaped MXFP4 MoE FFN (config 3 of the benchmark set: 4096 tokens,
 d_model 2880, 128 experts, top-4, W1 [128, 2880, 5760] and W2 [128, 2880, 2880] in MXFP4 with bf16 biases):
 router -> gather-GEMM (+bias, swiglu) -> scatter-GEMM (+bias, gate weight) -> top-k combine, on synthetic
 seeded inputs resident in HBM.  Prints ONE JSON line; `value` is the layer's TFLOP/s (2*R*K*N over both

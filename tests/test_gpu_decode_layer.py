@@ -2,7 +2,7 @@
 the three-call sequence it stands for (routing -> gather-GEMM + swiglu -> scatter-GEMM * gate -> combine).
 
 Routing decisions must be bit-equal to the oracle's (and the gate values close); the layer output is held to the same
-gates as the three-call layer tests.  Covers BASELINE config 4 at its real shape (128 experts, top-4, skewed router,
+gates as the three-call layer tests.  Covers benchmark config 4 at its real shape (128 experts, top-4, skewed router,
 T in {1, 4, 16, 64}), repeated launches on one workspace (the counters are left clean), heavy skew (one expert with
 many row blocks), odd shapes (K not a multiple of 128, the largest dimensions, more than 128 experts), and a HIP graph replayed with eager
 work in between."""

@@ -233,7 +233,7 @@ def _oracle_layer_on_active_experts(x, logits, k, W0):
 
 @pytest.mark.parametrize("T", [1, 4, 16, 64])
 def test_config4_full_shape_decode(api, device, gptoss_weights, T):
-    """BASELINE config 4 at its real shape: 128 experts, top-4, T in {1, 4, 16, 64}, router logits skewed by a
+    """Benchmark config 4 at its real shape: 128 experts, top-4, T in {1, 4, 16, 64}, router logits skewed by a
     per-expert bias N(0, 1.5), tiled MXFP4 weights with biases; the whole layer against the oracle."""
     g = torch.Generator().manual_seed(3)
     E, k, d = 128, 4, 2880
@@ -252,7 +252,7 @@ def test_config4_full_shape_decode(api, device, gptoss_weights, T):
 
 
 def test_config3_full_shape_sampled_tokens(api, device, gptoss_weights):
-    """BASELINE config 3 at its real shape (4096 tokens, 128 experts, top-4): the final output rows of 12 sampled
+    """Benchmark config 3 at its real shape (4096 tokens, 128 experts, top-4): the final output rows of 12 sampled
     tokens (the first four routed to experts 0, 63 and 127) against the oracle, which evaluates those tokens alone with
     the experts they use.  Covers the second GEMM, gate weights, scatter and combine at the full shape."""
     from oracle import routing as ort
@@ -474,7 +474,7 @@ def test_fused_combine_with_many_row_blocks_on_one_expert(api, device, gptoss_we
 
 
 def test_config5_full_shape_sampled_tokens(api, device):
-    """BASELINE config 5 at its real shape: the FINAL output rows of six sampled tokens, i.e. the second GEMM at
+    """Benchmark config 5 at its real shape: the FINAL output rows of six sampled tokens, i.e. the second GEMM at
     K = 14336 with per-token and per-channel scales, the gate weight, the scatter and the combine over the eight
     experts, against the oracle."""
     from triton_kernels.tensor import convert_layout, wrap_torch_tensor

@@ -1,6 +1,6 @@
 """GPU parity of the MX quantise / dequantise kernels (through the C ABI) against the CPU oracle.
 
-Cases mirror python/triton_kernels/tests/test_mxfp.py:92-291; the full BASELINE shape
+Cases mirror python/triton_kernels/tests/test_mxfp.py:92-291; the full benchmark shape
 [32, 2880, 5760] is checked through size-independent properties plus oracle comparison on slices."""
 import pytest
 import torch
