@@ -172,9 +172,12 @@ def test_baseline_shape_round_trip(mx, device):
 
 @pytest.mark.parametrize("M, K, view", [(37, 4096, "plain"), (5, 1000, "plain"), (9, 1003, "plain"), (6, 520, "offset"), (3, 7, "plain"),
                                         (4, 14336, "plain"), (3, 8256, "plain"), (2, 20000, "plain"),
-                                        # rows that are kept in registers between the two passes (2048 < K <= 4096, aligned), with a
-                                        # partly filled last vector, and the same length unaligned (two-pass kernel)
-                                        (5, 2056, "plain"), (3, 3000, "plain"), (3, 4096, "offset"), (3, 8192, "plain")])
+                                        # rows that a workgroup keeps in registers between the two passes (2048 < K <= 32768,
+                                        # aligned), with a partly filled last piece, and the same length unaligned (two-pass kernel)
+                                        (5, 2056, "plain"), (3, 3000, "plain"), (3, 4096, "offset"), (3, 8192, "plain"),
+                                        # long rows: eight pieces per thread up to 16384 elements, sixteen up to 32768, the two-pass
+                                        # kernel beyond
+                                        (2, 16384, "plain"), (3, 14344, "plain"), (2, 16392, "plain"), (2, 32768, "plain"), (2, 32776, "plain")])
 def test_quantize_fp8_rowwise_bit_exact(device, M, K, view):
     """Per-row e4m3 quantiser (the FP8 configuration's activation path): bytes bit-exact and scales equal to the
     oracle's, on rows that take the vector path, rows with a scalar tail, and rows that are not 16-byte aligned;

@@ -150,19 +150,23 @@ __global__ __launch_bounds__(256) void quant_fp8_rows_kernel(const uint16_t* x, 
 }
 
 // The same with the row held in registers between the two passes (rows 16-byte aligned, K a multiple of 8 and at most
-// NV * 512): one read of x instead of two.
+// NV * 2048): a WORKGROUP per row, NV 16-byte pieces per thread, the row maximum through LDS, one read of x instead of
+// two.  (With a wave per row and two passes some thirty rows per CU are between their passes at any time, 29 MB per XCD
+// at K = 14336 against an L2 of 4 MB, so the second pass came from memory again: 16384 x 14336 in 189 us, 134 us this
+// way.  A wave per row with the row in registers needs 4 NV registers per lane for a row four times as long per lane and
+// was slower than two passes from 8192 elements on; for rows of 4096 it took 25 us at 8192 rows, this takes 21.)
 template <int NV>
-__global__ __launch_bounds__(256) void quant_fp8_rows_reg_kernel(const uint16_t* x, int64_t stride_m, int64_t M, int64_t K, uint8_t* q,
-                                                                 int64_t stride_qm, float* scales) {
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= M) return;
+__global__ __launch_bounds__(256) void quant_fp8_rows_wg_kernel(const uint16_t* x, int64_t stride_m, int64_t M, int64_t K, uint8_t* q,
+                                                                int64_t stride_qm, float* scales) {
+  __shared__ float wmax_s[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x;
   const uint16_t* xr = x + row * stride_m;
   uint8_t* qr = q + row * stride_qm;
   uint4 v[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int64_t k = (int64_t)i * 512 + lane * 8;
+    const int64_t k = (int64_t)i * 2048 + tid * 8;
     v[i] = k < K ? *reinterpret_cast<const uint4*>(xr + k) : make_uint4(0u, 0u, 0u, 0u);
   }
   float m = 0.f;
@@ -174,12 +178,15 @@ __global__ __launch_bounds__(256) void quant_fp8_rows_reg_kernel(const uint16_t*
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  if (lane == 0) wmax_s[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(wmax_s[0], wmax_s[1]), fmaxf(wmax_s[2], wmax_s[3]));
   float s = m / 448.0f;
   if (s == 0.f) s = 1.0f;
-  if (lane == 0) scales[row] = s;
+  if (tid == 0) scales[row] = s;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    const int64_t k = (int64_t)i * 512 + lane * 8;
+    const int64_t k = (int64_t)i * 2048 + tid * 8;
     const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
     float q8[8];
 #pragma unroll
@@ -361,13 +368,16 @@ extern "C" int32_t tk_quant_fp8_rows(const void* x, int32_t dtype, int64_t M, in
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* xs = static_cast<const uint16_t*>(x);
   uint8_t* qd = static_cast<uint8_t*>(q);
-  // short aligned rows are kept in a wave's registers between the two passes and read once (measured at 8192 x 4096: 30 ->
-  // 25 us; with rows of 14336 the 128 registers a row needs leave too few waves to cover the conversion arithmetic, 200 ->
-  // 270 us, so longer rows take the two-pass kernel)
   const bool aligned = K % 8 == 0 && stride_m % 8 == 0 && stride_qm % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0;
-  if (aligned && K > 2048 && K <= 4096) {
-    hipLaunchKernelGGL(quant_fp8_rows_reg_kernel<8>, grid, block, 0, st, xs, stride_m, M, K, qd, stride_qm, scales);
-    return check_launch("quant_fp8_rows_reg_kernel");
+  if (aligned && K > 2048 && K <= 32768 && M <= 0x7FFFFFFF) {
+    const dim3 rows((unsigned)M);
+    if (K <= 4096)
+      hipLaunchKernelGGL(quant_fp8_rows_wg_kernel<2>, rows, block, 0, st, xs, stride_m, M, K, qd, stride_qm, scales);
+    else if (K <= 16384)
+      hipLaunchKernelGGL(quant_fp8_rows_wg_kernel<8>, rows, block, 0, st, xs, stride_m, M, K, qd, stride_qm, scales);
+    else
+      hipLaunchKernelGGL(quant_fp8_rows_wg_kernel<16>, rows, block, 0, st, xs, stride_m, M, K, qd, stride_qm, scales);
+    return check_launch("quant_fp8_rows_wg_kernel");
   }
   hipLaunchKernelGGL(quant_fp8_rows_kernel, grid, block, 0, st, xs, stride_m, M, K, qd, stride_qm, scales);
   return check_launch("quant_fp8_rows_kernel");
