@@ -115,16 +115,6 @@ __device__ __forceinline__ int row16_min_i32(int x) {
 #undef TK_STEP
   return x;
 }
-// inclusive prefix sum over the 64 lanes: four shifts inside the rows of 16, then the row totals are broadcast on
-__device__ __forceinline__ int wave_scan_i32(int x) {
-  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, true);  // row_shr:1
-  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, true);  // row_shr:2
-  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, true);  // row_shr:4
-  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, true);  // row_shr:8
-  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
-  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
-  return x;
-}
 __device__ __forceinline__ float row16_sum_f32(float v) {
   int x = __builtin_bit_cast(int, v);
 #define TK_STEP(ctrl) x = __builtin_bit_cast(int, __builtin_bit_cast(float, x) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false)));

@@ -64,6 +64,17 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
   return (a + b) + (c + d);
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP lane exchanges (no LDS round trips): four shifts inside the rows of 16,
+// then the row totals are broadcast on.  All 64 lanes must be active.
+__device__ __forceinline__ int wave_scan_i32(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, true);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, true);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, true);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, true);  // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
 // Top-k of one row spread over a wave: lane l holds the order-preserving keys of experts l, l + 64, ... in hi[]
 // (0 for columns past E).  Round j picks the largest key, ties to the lowest expert index (the reference packs
 // E_pad - idx under the key for the same effect, topk_details/_topk_forward.py:27-35,61), hands it to lane j and

@@ -220,14 +220,7 @@ __device__ __forceinline__ const int32_t* ragged_metadata(const int32_t* slice_s
 #pragma unroll
     for (int b = 0; b < kNumBlockSizes; ++b) v[1 + b] = (sz + ((1 << (kFirstBlockLog2 + b)) - 1)) >> (kFirstBlockLog2 + b);
 #pragma unroll
-    for (int q = 0; q < kQuantities; ++q) {
-      inc[q] = v[q];
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int o = __shfl_up(inc[q], off);
-        if (lane >= off) inc[q] += o;
-      }
-    }
+    for (int q = 0; q < kQuantities; ++q) inc[q] = wave_scan_i32(v[q]);  // (DPP: six lane exchanges through LDS each took 2 us more)
     __syncthreads();  // wave_tot may still be read by the previous trip
     if (lane == 63) {
 #pragma unroll
