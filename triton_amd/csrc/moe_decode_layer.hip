@@ -36,7 +36,6 @@ constexpr int kDecMaxUnits = 192;                      // units of one workgroup
 constexpr int kDecNW = 8;                              // waves per workgroup = K-slices of a unit
 constexpr int kDecXS = 3;                              // K-stages (of 128) per slice: K <= NW * XS * 128 = 3072
 constexpr int kDecRing = 3;                            // units of weight blocks a wave holds or has requested
-constexpr int kDecMaskWords = kDecMaxRows / 32;        // token bits per expert (T <= 256)
 constexpr int kDecBlockStride = 32;                    // words between two row blocks' counters (a cache line each)
 constexpr int kDecBlockWords = (kDecMaxRows + kDecMaxRows / 16) * kDecBlockStride;  // 16-row blocks: at most min(E, R) + R / 16
 
@@ -90,38 +89,6 @@ __device__ long long dec_stamps[1024][20];
 #define DEC_UNIT_STAMP(i) do {} while (0)
 #define DEC_STAMP(n) do {} while (0)
 #endif
-
-// reductions inside a DPP row of 16 lanes (every lane of the row ends up with the row's result)
-#define TK_ROW16(OP)                                                                                   \
-  OP(TK_DPP_QUAD_XOR1) OP(TK_DPP_QUAD_XOR2) OP(TK_DPP_ROW_HALF_MIRROR) OP(TK_DPP_ROW_MIRROR)
-__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
-  int x = (int)v;
-#define TK_STEP(ctrl)                                                                                   \
-  {                                                                                                     \
-    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false);             \
-    x = (int)(o > (uint32_t)x ? o : (uint32_t)x);                                                       \
-  }
-  TK_ROW16(TK_STEP)
-#undef TK_STEP
-  return (uint32_t)x;
-}
-__device__ __forceinline__ int row16_min_i32(int x) {
-#define TK_STEP(ctrl)                                                                                   \
-  {                                                                                                     \
-    const int o = __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false);                            \
-    x = o < x ? o : x;                                                                                  \
-  }
-  TK_ROW16(TK_STEP)
-#undef TK_STEP
-  return x;
-}
-__device__ __forceinline__ float row16_sum_f32(float v) {
-  int x = __builtin_bit_cast(int, v);
-#define TK_STEP(ctrl) x = __builtin_bit_cast(int, __builtin_bit_cast(float, x) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false)));
-  TK_ROW16(TK_STEP)
-#undef TK_STEP
-  return __builtin_bit_cast(float, x);
-}
 
 constexpr int kThrough = 1 | 16;  // aux bits of the buffer instructions: sc0 | sc1 (write through / read around the L2)
 
@@ -192,23 +159,7 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       uint32_t sel_key[2] = {0u, 0u};
       int sel_idx[2] = {0, 0};
       uint32_t key0 = 0;
-      for (int j = 0; j < k; ++j) {
-        uint32_t m = 0;
-#pragma unroll
-        for (int i = 0; i < VPL; ++i) m = (!((ret >> i) & 1u) && key[i] > m) ? key[i] : m;
-        m = row16_max_u32(m);
-        int idx = 0x7FFFFFFF;
-#pragma unroll
-        for (int i = VPL - 1; i >= 0; --i) idx = (!((ret >> i) & 1u) && key[i] == m) ? l16 * VPL + i : idx;
-        idx = row16_min_i32(idx);
-        const int mine = idx - l16 * VPL;
-        if (mine >= 0 && mine < VPL) ret |= 1u << mine;
-        if (j == 0) key0 = m;
-        if ((j & 15) == l16) {
-          sel_key[j >> 4] = m;
-          sel_idx[j >> 4] = idx;
-        }
-      }
+      row16_topk<VPL>(key, ret, k, l16, sel_key, sel_idx, key0);
       if (row0 == 0) DEC_STAMP(19);
       // softmax over the k kept logits (fp32): z = exp(v - max) / sum
       float outv[2], z[2];
@@ -557,7 +508,6 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
     const int cnt = hist_s[e];
     const int row0 = offs_s[e] + rb * 16;                       // first expert-sorted row of the block
     const int rows = cnt - rb * 16 < 16 ? cnt - rb * 16 : 16;  // valid rows of the block
-    const int K = ph == 2 ? p.K2 : p.K1;
     if (i == 1) DEC_STAMP(3);
     if (i == n1) DEC_STAMP(4);
     if (cur.key != cur_key) {

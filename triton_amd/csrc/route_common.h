@@ -75,6 +75,69 @@ __device__ __forceinline__ int wave_scan_i32(int x) {
   x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
   return x;
 }
+// reductions inside a DPP row of 16 lanes (every lane of the row ends up with the row's result)
+#define TK_ROW16(OP)                                                                                   \
+  OP(TK_DPP_QUAD_XOR1) OP(TK_DPP_QUAD_XOR2) OP(TK_DPP_ROW_HALF_MIRROR) OP(TK_DPP_ROW_MIRROR)
+__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
+  int x = (int)v;
+#define TK_STEP(ctrl)                                                                                   \
+  {                                                                                                     \
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false);             \
+    x = (int)(o > (uint32_t)x ? o : (uint32_t)x);                                                       \
+  }
+  TK_ROW16(TK_STEP)
+#undef TK_STEP
+  return (uint32_t)x;
+}
+__device__ __forceinline__ int row16_min_i32(int x) {
+#define TK_STEP(ctrl)                                                                                   \
+  {                                                                                                     \
+    const int o = __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false);                            \
+    x = o < x ? o : x;                                                                                  \
+  }
+  TK_ROW16(TK_STEP)
+#undef TK_STEP
+  return x;
+}
+__device__ __forceinline__ float row16_sum_f32(float v) {
+  int x = __builtin_bit_cast(int, v);
+#define TK_STEP(ctrl) x = __builtin_bit_cast(int, __builtin_bit_cast(float, x) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, x, ctrl, 0xF, 0xF, false)));
+  TK_ROW16(TK_STEP)
+#undef TK_STEP
+  return __builtin_bit_cast(float, x);
+}
+
+
+// Top-k of FOUR rows at a time in one wave: the sixteen lanes of a DPP row own one row of logits, lane l of the row the
+// VPL consecutive experts l * VPL .. l * VPL + VPL - 1 as order-preserving keys (`retired` bit i: key[i] is out of the
+// running, columns past E from the start).  A round = the row's largest key still in the running (in-lane maximum,
+// then four DPP steps inside the row) and the LOWEST expert index holding it (the same again with a minimum): ties go
+// to the lower expert, as the reference's packed sort key does (topk_details/_topk_forward.py:27-35,61).  Round j's
+// winner lands in lane j & 15 of the row, slot j >> 4 (k <= 32); key0 = the first round's key (the row maximum).  No
+// lane leaves its row, so the four rows cost what one costs.
+template <int VPL>
+__device__ __forceinline__ void row16_topk(const uint32_t (&key)[VPL], uint32_t retired, int k, int l16, uint32_t (&sel_key)[2],
+                                           int (&sel_idx)[2], uint32_t& key0) {
+  uint32_t ret = retired;
+  for (int j = 0; j < k; ++j) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) m = (!((ret >> i) & 1u) && key[i] > m) ? key[i] : m;
+    m = row16_max_u32(m);
+    int idx = 0x7FFFFFFF;
+#pragma unroll
+    for (int i = VPL - 1; i >= 0; --i) idx = (!((ret >> i) & 1u) && key[i] == m) ? l16 * VPL + i : idx;
+    idx = row16_min_i32(idx);
+    const int mine = idx - l16 * VPL;
+    if (mine >= 0 && mine < VPL) ret |= 1u << mine;
+    if (j == 0) key0 = m;
+    if ((j & 15) == l16) {
+      sel_key[j >> 4] = m;
+      sel_idx[j >> 4] = idx;
+    }
+  }
+}
+
 // Top-k of one row spread over a wave: lane l holds the order-preserving keys of experts l, l + 64, ... in hi[]
 // (0 for columns past E).  Round j picks the largest key, ties to the lowest expert index (the reference packs
 // E_pad - idx under the key for the same effect, topk_details/_topk_forward.py:27-35,61), hands it to lane j and

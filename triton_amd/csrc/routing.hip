@@ -574,7 +574,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
   __shared__ __attribute__((aligned(16))) int32_t eid_s[kSmallEntries];
   __shared__ uint32_t val_s[kSmallEntries];
   __shared__ int32_t hist_s[kMaxExperts];
-  __shared__ uint32_t words_s[kScanWaves][EPL * 2];
+  __shared__ uint32_t words_s[kScanWaves][4 * EPL * 2];  // bitmatrix words of the rows a wave has in hand (up to four)
   const TopkParams& p = q.t;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int E = p.E, k = p.k, T = p.T;
@@ -587,6 +587,91 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
   // ---- phase 1: top-k per row (wave w takes rows w, w + 16, ...); the next row's logits are fetched while the
   // current row is selected, so a wave pays the memory latency once ----
   // (rows in batches, all loads of a batch in flight together and none inside the per-row code: see route_topk_kernel)
+  constexpr bool kRows4 = !PROVIDED && EPL <= 8;  // (up to 512 experts: a lane holds at most 32 keys)
+  // (with more rows than waves only; and k <= 16, where the gate values come out bit for bit as from the row-per-wave
+  // code below: the sums meet the same values in the same lanes of a DPP row)
+  bool rows4 = false;
+  if constexpr (kRows4) rows4 = k <= 16 && T > kScanWaves && n_rows > kScanWaves;
+  if constexpr (kRows4) if (rows4) {
+    // FOUR rows per wave at a time: the sixteen lanes of a DPP row own a row (row16_topk), so 64 rows are in hand per
+    // pass of the sixteen waves instead of 16, and a wave's pass costs what one row cost (about 1.7 us); the next
+    // pass's logits are fetched before this pass's rows are selected.
+    constexpr int VPL = EPL * 4, W = EPL * 2;
+    const int l16 = lane & 15, sub = lane >> 4;
+    const int n_live = T < n_rows ? T : n_rows;
+    float cur[VPL], nxt[VPL];
+    auto fetch = [&](int r, float (&dst)[VPL]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int e = l16 * VPL + i;
+        dst[i] = (r < n_live && e < E) ? load_logit<DT>(p.logits, (int64_t)r * p.stride_m + e) : 0.f;
+      }
+    };
+    fetch(wave * 4 + sub, cur);
+    for (int row0 = 0; row0 + wave * 4 < n_live; row0 += kScanWaves * 4) {
+      const int row = row0 + wave * 4 + sub;
+      const bool row_ok = row < n_live;
+      fetch(row + kScanWaves * 4, nxt);
+      uint32_t key[VPL];
+      uint32_t retired = 0;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        key[i] = ordered_key(cur[i]);
+        retired |= (l16 * VPL + i >= E ? 1u : 0u) << i;
+      }
+      uint32_t sel_key[2] = {0u, 0u};
+      int sel_idx[2] = {0x7FFFFFFF, 0x7FFFFFFF};
+      uint32_t key0 = 0;
+      row16_topk<VPL>(key, retired, k, l16, sel_key, sel_idx, key0);
+      float outv[2], z[2];
+      const float vmax = key_to_float(key0);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        outv[h] = key_to_float(sel_key[h]);
+        z[h] = l16 + 16 * h < k ? expf(outv[h] - vmax) : 0.f;
+      }
+      if (p.apply_softmax) {
+        const float sum = row16_sum_f32(z[0] + z[1]);
+        outv[0] = z[0] / sum;
+        outv[1] = z[1] / sum;
+      }
+      if (p.bitmatrix) {
+        if (l16 < words) words_s[wave][sub * W + l16] = 0u;
+        wave_sync();
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int j = l16 + 16 * h;
+        if (row_ok && j < k) {
+          const int myidx = sel_idx[h];
+          const bool live = myidx >= 0 && myidx < E;
+          if (p.vals) store_val<DT>(p.vals, (int64_t)row * k + j, outv[h]);
+          p.indx[(int64_t)row * k + j] = (int16_t)(live ? myidx : -1);
+          eid_s[row * k + j] = live ? myidx : -1;
+          uint32_t bits;  // the gate value as it is stored (bits of the logits dtype)
+          if (DT == TK_F32)
+            bits = f32_bits(outv[h]);
+          else if (DT == TK_BF16)
+            bits = f32_to_bf16_bits(outv[h]);
+          else
+            bits = f32_to_f16_bits(outv[h]);
+          val_s[row * k + j] = bits;
+          if (live) {
+            atomicAdd(&hist_s[myidx], 1);
+            if (p.bitmatrix) atomicOr(&words_s[wave][sub * W + (myidx >> 5)], 1u << (myidx & 31));
+          }
+        }
+      }
+      if (p.bitmatrix) {
+        wave_sync();
+        if (row_ok && l16 < words) p.bitmatrix[(int64_t)l16 * p.bm_stride_w + row] = words_s[wave][sub * W + l16];
+        wave_sync();
+      }
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) cur[i] = nxt[i];
+    }
+  }
+  if (!rows4) {
   constexpr int kBatch = EPL <= 2 ? 4 : EPL <= 8 ? 2 : 1;
   float nv[kBatch][EPL];
   for (int row0 = wave; row0 < T && row0 < n_rows; row0 += kScanWaves * kBatch) {
@@ -661,6 +746,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
       if (lane < words) p.bitmatrix[(int64_t)lane * p.bm_stride_w + row] = words_s[wave][lane];
       wave_sync();
     }
+  }
   }
   }
   __syncthreads();
