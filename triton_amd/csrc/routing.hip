@@ -101,12 +101,13 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
 #pragma unroll
     for (int r = 0; r < kBatch; ++r) {
       const int row = row0 + r;
-      if (row < row_end && row < n_rows) {
+      // (no conditions around the loads: rows past the run repeat its last row and are never used, columns past E the
+      // last column and their keys are retired; behind a condition every load of a 16-bit row got a wait of its own)
+      const int64_t at = (int64_t)(row < row_end ? row : row_end - 1) * p.stride_m;
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) {
-          const int e = lane + 64 * i;
-          batch_v[r][i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
-        }
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        batch_v[r][i] = load_logit<DT>(p.logits, at + (e < E ? e : E - 1));
       }
     }
   }
@@ -600,11 +601,14 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
     const int l16 = lane & 15, sub = lane >> 4;
     const int n_live = T < n_rows ? T : n_rows;
     float cur[VPL], nxt[VPL];
+    // (loads without conditions: a row past the last repeats the last row, a column past E the last column; their keys
+    // are retired or their rows never written.  Behind a condition each load got a branch and a wait of its own.)
     auto fetch = [&](int r, float (&dst)[VPL]) __attribute__((always_inline)) {
+      const int64_t at = (int64_t)(r < T ? r : T - 1) * p.stride_m;
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
         const int e = l16 * VPL + i;
-        dst[i] = (r < n_live && e < E) ? load_logit<DT>(p.logits, (int64_t)r * p.stride_m + e) : 0.f;
+        dst[i] = load_logit<DT>(p.logits, at + (e < E ? e : E - 1));
       }
     };
     fetch(wave * 4 + sub, cur);
@@ -679,12 +683,13 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
 #pragma unroll
     for (int r = 0; r < kBatch; ++r) {
       const int row = row0 + r * kScanWaves;
-      if (row < T && row < n_rows) {
+      // (no conditions around the loads: rows past the last repeat the last row and are never used, columns past E
+      // the last column and their keys are retired; behind a condition every load of a 16-bit row got a wait of its own)
+      const int64_t at = (int64_t)(row < T ? row : T - 1) * p.stride_m;
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) {
-          const int e = lane + 64 * i;
-          nv[r][i] = e < E ? load_logit<DT>(p.logits, (int64_t)row * p.stride_m + e) : 0.f;
-        }
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        nv[r][i] = load_logit<DT>(p.logits, at + (e < E ? e : E - 1));
       }
     }
   }
