@@ -111,6 +111,20 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
       }
     }
   }
+  // The keys of the whole batch are taken HERE, in front of the first row's stores.  Loads and stores of a wave complete
+  // in order and share one counter, the stores below sit behind conditions, so the compiler counts none of them: a wait
+  // for a later row's logits placed behind an earlier row's stores waits for those stores as well, a memory round trip
+  // per row.
+  uint32_t bkey[kBatch][EPL];
+  if constexpr (!PROVIDED) {
+#pragma unroll
+    for (int r = 0; r < kBatch; ++r)
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        bkey[r][i] = lane + 64 * i < E ? ordered_key(batch_v[r][i]) : 0u;
+        asm volatile("" ::"v"(bkey[r][i]) : "memory");
+      }
+  }
 #pragma unroll
   for (int r = 0; r < kBatch; ++r) {
     const int row = row0 + r;
@@ -123,10 +137,7 @@ __global__ __launch_bounds__(kWaves * 64) void route_topk_kernel(const TopkParam
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
       }
     } else {
-      uint32_t key[EPL];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(batch_v[r][i]) : 0u;
-      wave_topk<EPL>(key, k, E, lane, myval, myidx);
+      wave_topk<EPL>(bkey[r], k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
@@ -556,6 +567,11 @@ __global__ __launch_bounds__(kScanThreads) void ragged_remap_kernel(const RemapP
 // reads, all lanes reading the same address), and the ragged metadata follows.  One launch instead of three:
 // at decode batch sizes the pass is pure launch latency.
 constexpr int kSmallEntries = 1024;
+// ... and is USED up to this many entries: the single workgroup is bound by one CU's instruction rate (sixteen waves share
+// four SIMDs), so its top-k phase grows with the batch (inside the launch 6.6 us at 64 entries, 9.9 at 256, 22.7 at 1024)
+// while the three kernels, spread over the chip, stay at 20 us from launch to end: at 384 / 512 / 768 / 1024 entries a
+// replayed graph measured 24.8 / 27.2 / 34.4 / 42.6 us for the single launch against 19.8 / 20.5 / 19.8 / 20.5.
+constexpr int kSmallCut = 256;
 
 struct SmallParams {
   TopkParams t;
@@ -612,17 +628,17 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
       }
     };
     fetch(wave * 4 + sub, cur);
+    uint32_t key[VPL];
+    uint32_t retired = 0;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      key[i] = ordered_key(cur[i]);
+      retired |= (l16 * VPL + i >= E ? 1u : 0u) << i;
+    }
     for (int row0 = 0; row0 + wave * 4 < n_live; row0 += kScanWaves * 4) {
       const int row = row0 + wave * 4 + sub;
       const bool row_ok = row < n_live;
       fetch(row + kScanWaves * 4, nxt);
-      uint32_t key[VPL];
-      uint32_t retired = 0;
-#pragma unroll
-      for (int i = 0; i < VPL; ++i) {
-        key[i] = ordered_key(cur[i]);
-        retired |= (l16 * VPL + i >= E ? 1u : 0u) << i;
-      }
       uint32_t sel_key[2] = {0u, 0u};
       int sel_idx[2] = {0x7FFFFFFF, 0x7FFFFFFF};
       uint32_t key0 = 0;
@@ -638,6 +654,14 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
         const float sum = row16_sum_f32(z[0] + z[1]);
         outv[0] = z[0] / sum;
         outv[1] = z[1] / sum;
+      }
+      // The next pass's keys are taken HERE, in front of this pass's stores.  Loads and stores of a wave complete in
+      // order and share one counter, the stores below sit behind conditions, so the compiler counts none of them: a
+      // wait for these loads placed behind the stores would wait for every store as well, a memory round trip per pass.
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        key[i] = ordered_key(nxt[i]);
+        asm volatile("" ::"v"(key[i]) : "memory");
       }
       if (p.bitmatrix) {
         if (l16 < words) words_s[wave][sub * W + l16] = 0u;
@@ -671,8 +695,6 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
         if (row_ok && l16 < words) p.bitmatrix[(int64_t)l16 * p.bm_stride_w + row] = words_s[wave][sub * W + l16];
         wave_sync();
       }
-#pragma unroll
-      for (int i = 0; i < VPL; ++i) cur[i] = nxt[i];
     }
   }
   if (!rows4) {
@@ -693,6 +715,20 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
       }
     }
   }
+  // The keys of the whole batch are taken HERE, in front of the first row's stores.  Loads and stores of a wave complete
+  // in order and share one counter, the stores below sit behind conditions, so the compiler counts none of them: a wait
+  // for a later row's logits placed behind an earlier row's stores waits for those stores as well, a memory round trip
+  // per row.
+  uint32_t bkey[kBatch][EPL];
+  if constexpr (!PROVIDED) {
+#pragma unroll
+    for (int r = 0; r < kBatch; ++r)
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        bkey[r][i] = lane + 64 * i < E ? ordered_key(nv[r][i]) : 0u;
+        asm volatile("" ::"v"(bkey[r][i]) : "memory");
+      }
+  }
 #pragma unroll
   for (int r = 0; r < kBatch; ++r) {
     const int row = row0 + r * kScanWaves;
@@ -705,10 +741,7 @@ __global__ __launch_bounds__(kScanThreads) void route_small_kernel(const SmallPa
         if (p.logits && myidx >= 0) myval = load_logit<DT>(p.logits, (int64_t)row * p.stride_m + myidx);
       }
     } else {
-      uint32_t key[EPL];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? ordered_key(nv[r][i]) : 0u;
-      wave_topk<EPL>(key, k, E, lane, myval, myidx);
+      wave_topk<EPL>(bkey[r], k, E, lane, myval, myidx);
     }
     float outv = myval;
     if (p.apply_softmax) {
@@ -991,7 +1024,7 @@ static int32_t route_impl(const tk_route_desc* d, void* workspace, tk_stream_t s
   tp.fill_a = want_meta ? d->col_sorted_indx : nullptr;
   tp.fill_b = want_meta ? d->row_sorted_indx : nullptr;
   tp.fill_c = want_meta ? d->gather_indx : nullptr;
-  if ((int64_t)T * k <= kSmallEntries) {
+  if ((int64_t)T * k <= kSmallCut) {
     // small batch: the whole pass in one launch
     SmallParams sq;
     sq.t = tp;
