@@ -154,7 +154,8 @@ extern "C" int32_t tk_moe_gemm(const tk_gemm_desc* d, tk_stream_t stream) {
       const int64_t y_rows = d->scatter_indx ? d->scatter_len : d->M;
       const int64_t elem = mx_out ? 1 : 2, piece = swiglu ? 4 : 8;
       const int64_t y_bytes = y_rows * d->y_stride_m * elem;
-      bool fast = x_rows > 0 && x_rows * d->x_stride_m < ((int64_t)1 << 32) && x_rows * d->xs_stride_m < ((int64_t)1 << 32) && d->x_stride_m >= 0 &&
+      // (K >= 512: the persistent form reads a row's activation scales sixteen at a time)
+      bool fast = d->K >= 512 && x_rows > 0 && x_rows * d->x_stride_m < ((int64_t)1 << 32) && x_rows * d->xs_stride_m < ((int64_t)1 << 32) && d->x_stride_m >= 0 &&
                   d->xs_stride_m >= 0 && !extras && d->n_slices <= kMetaSlices && y_bytes > 0 && y_bytes < ((int64_t)1 << 31) && d->y_stride_m >= 0;
       if (mx_out)
         fast = fast && p.y_vec && y_rows * d->ys_stride_m < ((int64_t)1 << 31) && d->ys_stride_m >= 0;

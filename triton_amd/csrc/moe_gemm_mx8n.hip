@@ -620,8 +620,10 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
 
   typename FR::acc_t acc[NFW][MFW];
   u32x4_t xreg[XD][XCH];
-  uint32_t xsreg[XD] = {};
-  int xsshift[XD] = {};
+  // the activation scales of this thread's row for FOUR stages (16 blocks of 32) at a time: the group in use and the one
+  // after it, and by how many bytes each load was moved back to stay inside the row (the last group of a row)
+  u32x4_t xsq_cur = {}, xsq_nxt = {};
+  int gsh_cur = 0, gsh_nxt = 0;
   u32x4_t wraw[WD][NFW][NS];
   uint32_t sd[WD][NFW];
   i32x8_t xf[2][MFW];
@@ -632,21 +634,27 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
     k0 = k0 < K - 16 ? k0 : K - 16;
     xreg[slot][j] = *reinterpret_cast<const u32x4_t*>(p.x + (xoff[j] + (uint32_t)k0));
   };
-  auto load_x_scale = [&](int s, int slot) __attribute__((always_inline)) {
-    int b0 = s * 4;
-    b0 = b0 < kblocks - 4 ? b0 : kblocks - 4;
-    uint32_t v;
-    __builtin_memcpy(&v, p.x_mx_scale + (xsoff + (uint32_t)b0), 4);
-    xsreg[slot] = v;
-    xsshift[slot] = s * 4 - b0;
+  // One 16-byte load per row and four stages instead of a 4-byte load per row and stage: every lane of such a load owns
+  // another row, i.e. another cache line, so the scales, 4 bytes per row and stage, cost as many line look-ups per
+  // stage as the 128 bytes of activations per row that they belong to.  (kblocks >= 16: the host's condition.)
+  auto load_x_scale_group = [&](int g, u32x4_t& dst, int& gsh) __attribute__((always_inline)) {
+    int b0 = g * 16;
+    b0 = b0 < kblocks - 16 ? b0 : kblocks - 16;
+    __builtin_memcpy(&dst, p.x_mx_scale + (xsoff + (uint32_t)b0), 16);
+    gsh = g * 16 - b0;
   };
   auto store_x_piece = [&](int j, int buf, int slot) __attribute__((always_inline)) {
     *reinterpret_cast<u32x4_t*>(lds + buf * XBYTES + xlds0 + j * 32 * XPITCH) = xreg[slot][j];
   };
-  auto store_x_scale = [&](int buf, int slot) __attribute__((always_inline)) {
-    const int sh = xsshift[slot] < 4 ? xsshift[slot] : 4;
-    const uint64_t wide = ((uint64_t)0x7F7F7F7Fu << 32) | xsreg[slot];
-    const uint32_t v = (uint32_t)(wide >> (8 * sh));
+  // stage d (0..3) of the group held in q: its four scale bytes start 4 d + gsh bytes into q; bytes past q are 2^0
+  auto store_x_scale = [&](int buf, const u32x4_t& q, int gsh, int d) __attribute__((always_inline)) {
+    const int o = 4 * d + gsh;
+    const int idx = o >> 2, sh = (o & 3) * 8;
+    auto word = [&](int i) __attribute__((always_inline)) -> uint32_t {
+      return i == 0 ? q.x : i == 1 ? q.y : i == 2 ? q.z : i == 3 ? q.w : 0x7F7F7F7Fu;
+    };
+    const uint64_t wide = ((uint64_t)word(idx + 1) << 32) | word(idx);
+    const uint32_t v = (uint32_t)(wide >> sh);
     // (no branch inside the K loop: threads past the tile's rows write into the unused pad bytes of a row)
     const int at = tid < BM ? tid * XPITCH + KC : (tid - BM) * XPITCH + KC + 4;
     *reinterpret_cast<uint32_t*>(lds + buf * XBYTES + at) = v;
@@ -705,8 +713,19 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
           }
         } else if constexpr (o == 2 * NJ) {
           if constexpr (q == 0) {
-            store_x_scale(PAR ^ 1, XS);
-            load_x_scale(c + 1 + XD, XS);
+            // stage c + 1's scales go to LDS; c is a multiple of UNR = 4 at unroll position 0, so stage c + 1 is stage
+            // (WSU + 1) % 4 of its group.  Position 0 takes over the group requested at position 1 of the round before,
+            // position 3 already serves the next round's first stage from it.
+            constexpr int D = (WSU + 1) & 3;
+            if constexpr (WSU == 0) {
+              xsq_cur = xsq_nxt;
+              gsh_cur = gsh_nxt;
+            }
+            if constexpr (D == 0)
+              store_x_scale(PAR ^ 1, xsq_nxt, gsh_nxt, 0);
+            else
+              store_x_scale(PAR ^ 1, xsq_cur, gsh_cur, D);
+            if constexpr (WSU == 1) load_x_scale_group((c + 3) >> 2, xsq_nxt, gsh_nxt);
           }
         } else {
           if constexpr (q == 0) load_w(WSL{}, c + WD - 1);
@@ -735,7 +754,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
   // previous unit's epilogue arithmetic
   auto first_loads = [&]() __attribute__((always_inline)) {
     static_for<0, XCH>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, 0, 0); });
-    load_x_scale(0, 0);
+    load_x_scale_group(0, xsq_nxt, gsh_nxt);
     __builtin_amdgcn_sched_barrier(0);
     load_w(S0, 0);
     __builtin_amdgcn_sched_barrier(0);
@@ -750,7 +769,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
     // the loads left in flight at the loop header are in the order the steady state leaves them in at the top of a
     // stage: activations, their scales, weights of stage 1, then of stage 2
     static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { store_x_piece(decltype(jc)::value, 0, 0); });
-    store_x_scale(0, 0);
+    store_x_scale(0, xsq_nxt, gsh_nxt, 0);
+    xsq_cur = xsq_nxt;
+    gsh_cur = gsh_nxt;
     __builtin_amdgcn_sched_barrier(0);
     // what the stages -max(XD, WD - 2) .. -1 would have issued had the loop been running: stage i requests the activations
     // of stage i + 1 + XD, then the weights of stage i + WD - 1 (this unit's: indices from 1 on)
@@ -760,7 +781,6 @@ __global__ __launch_bounds__(256) void moe_gemm_mx8p_kernel(const GemmParams p) 
       constexpr int sx = i + 1 + XD, sw = i + WD - 1;
       if constexpr (sx >= 1) {
         static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) { load_x_piece(decltype(jc)::value, sx, sx % XD); });
-        load_x_scale(sx, sx % XD);
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (sw >= 1) {
