@@ -92,7 +92,10 @@ __device__ long long dec_stamps[1024][20];
 
 constexpr int kThrough = 1 | 16;  // aux bits of the buffer instructions: sc0 | sc1 (write through / read around the L2)
 
-template <int VPL>
+// ONCE: no expert has more than one row block (the host knows it from T <= 16: a token's k experts differ), so every
+// weight byte is read exactly once by the whole grid and is fetched with the non-temporal hint; with several row
+// blocks on an expert the later ones find the fragment in the L2 and the hint would take that away.
+template <int VPL, bool ONCE>
 __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void moe_decode_layer_kernel(const DecodeParams p) {
   constexpr int NW = kDecNW, XS = kDecXS, NT = NW * 64;
   typedef Frag<16> FR;
@@ -343,8 +346,15 @@ __global__ __launch_bounds__(kDecNW * 64) __attribute__((amdgpu_waves_per_eu(2, 
       // (global address space spelled out: the pointers come out of the LDS table, the compiler takes them for generic
       // ones, and with FLAT loads in flight every wait for memory on this target is a wait for ALL of it, i.e. the ring
       // of weight blocks would be drained at the head of every unit)
-      wr[H][j][g] = *(const __attribute__((address_space(1))) u32x4_t*)(u.w + (int64_t)s * 2048 + g * 256 + wlane);
-      sr[H][j][g] = *(const __attribute__((address_space(1))) uint32_t*)(u.s + (int64_t)s * 128 + g * 64 + slane);
+      const auto* wp = (const __attribute__((address_space(1))) u32x4_t*)(u.w + (int64_t)s * 2048 + g * 256 + wlane);
+      const auto* sp = (const __attribute__((address_space(1))) uint32_t*)(u.s + (int64_t)s * 128 + g * 64 + slane);
+      if constexpr (ONCE) {
+        wr[H][j][g] = __builtin_nontemporal_load(wp);
+        sr[H][j][g] = __builtin_nontemporal_load(sp);
+      } else {
+        wr[H][j][g] = *wp;
+        sr[H][j][g] = *sp;
+      }
     }
   };
   auto unit_nst = [&](const DecUnit& u) __attribute__((always_inline)) -> int { return (u.key >> 24) == 2 ? p.nst2 : p.nst1; };
@@ -719,7 +729,7 @@ int resident_workgroups() {
   int n = cached[dev].load(std::memory_order_relaxed);
   if (n == 0) {
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(moe_decode_layer_kernel<VPL>), kDecNW * 64, 0) != hipSuccess || per_cu <= 0)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(moe_decode_layer_kernel<VPL, false>), kDecNW * 64, 0) != hipSuccess || per_cu <= 0)
       return 0;
     per_cu = 1;  // (a wave holds up to two units of weight blocks in its registers: one workgroup fills a CU)
     n = per_cu * device_cu_count();
@@ -829,9 +839,19 @@ extern "C" int32_t tk_moe_decode_layer(const tk_decode_layer_desc* d, tk_stream_
   if (max_blocks * (p.nfr1 + p.nfr2) / grid + 4 > kDecMaxUnits)
     return fail(TK_ERR_UNSUPPORTED, "tk_moe_decode_layer: %lld row blocks x %d fragments over %d workgroups exceed the kernel's unit table", (long long)max_blocks, p.nfr1 + p.nfr2, grid);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (small_e)
-    hipLaunchKernelGGL(moe_decode_layer_kernel<8>, dim3((unsigned)grid), dim3(kDecNW * 64), 0, st, p);
-  else
-    hipLaunchKernelGGL((moe_decode_layer_kernel<kDecMaxExperts / 16>), dim3((unsigned)grid), dim3(kDecNW * 64), 0, st, p);
+  const bool once = T <= 16;  // at most 16 rows, i.e. one row block, per expert: measured 43.0 -> 41.5 us at T = 4, 63.9 -> 61.1 at 16
+                              // (gpt-oss shape), and 102 -> 107 us at T = 64 with skewed routing, hence the switch
+  const dim3 g((unsigned)grid), b(kDecNW * 64);
+  if (small_e) {
+    if (once)
+      hipLaunchKernelGGL((moe_decode_layer_kernel<8, true>), g, b, 0, st, p);
+    else
+      hipLaunchKernelGGL((moe_decode_layer_kernel<8, false>), g, b, 0, st, p);
+  } else {
+    if (once)
+      hipLaunchKernelGGL((moe_decode_layer_kernel<kDecMaxExperts / 16, true>), g, b, 0, st, p);
+    else
+      hipLaunchKernelGGL((moe_decode_layer_kernel<kDecMaxExperts / 16, false>), g, b, 0, st, p);
+  }
   return check_launch("moe_decode_layer_kernel");
 }
