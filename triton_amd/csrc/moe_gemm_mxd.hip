@@ -129,7 +129,9 @@ __device__ __forceinline__ void combine_epilogue(const GemmParams& p, f32x4_t (&
     }
 }
 
-template <int MR, int NFD, bool SWIGLU>
+// ONCE: the whole problem is one row block per slice (at most 16 rows in all), so every weight byte is read exactly
+// once and is fetched with the non-temporal hint; several row blocks of a slice share its fragments through the L2.
+template <int MR, int NFD, bool SWIGLU, bool ONCE = false>
 __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   typedef Frag<16> FR;
   constexpr int WDD = 4, XDD = 4;  // ring depths (stages) of the weight / activation registers (both run 3 stages ahead)
@@ -232,8 +234,15 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
     for (int fd = 0; fd < NFD; ++fd)
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
-        wr[SL][fd][g] = *reinterpret_cast<const u32x4_t*>(wbase[fd] + (int64_t)s * 2048 + g * 256);
-        sr[SL][fd][g] = *reinterpret_cast<const uint32_t*>(sbase[fd] + (int64_t)s * 128 + g * 64);
+        const u32x4_t* wp = reinterpret_cast<const u32x4_t*>(wbase[fd] + (int64_t)s * 2048 + g * 256);
+        const uint32_t* sp = reinterpret_cast<const uint32_t*>(sbase[fd] + (int64_t)s * 128 + g * 64);
+        if constexpr (ONCE) {
+          wr[SL][fd][g] = __builtin_nontemporal_load(wp);
+          sr[SL][fd][g] = __builtin_nontemporal_load(sp);
+        } else {
+          wr[SL][fd][g] = *wp;
+          sr[SL][fd][g] = *sp;
+        }
       }
   };
   auto load_x = [&](auto slot_c, int i) __attribute__((always_inline)) {
@@ -343,7 +352,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mxd_kernel(const GemmParams p) {
   }
 }
 
-template <int MR, int NFD>
+template <int MR, int NFD, bool ONCE = false>
 int32_t launch_mxd_n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st) {
   GemmParams q = p;
   q.total_tiles = grid_m;  // row blocks in the non-ragged case
@@ -352,9 +361,9 @@ int32_t launch_mxd_n(const GemmParams& p, int grid_m, bool swiglu, hipStream_t s
   if (grid <= 0) return TK_OK;
   if (grid > 0x7FFFFFFF) return fail(TK_ERR_UNSUPPORTED, "tk_moe_gemm: grid too large");
   if (swiglu)
-    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, true>), dim3((unsigned)grid), dim3(256), 0, st, q);
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, true, ONCE>), dim3((unsigned)grid), dim3(256), 0, st, q);
   else
-    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, false>), dim3((unsigned)grid), dim3(256), 0, st, q);
+    hipLaunchKernelGGL((moe_gemm_mxd_kernel<MR, NFD, false, ONCE>), dim3((unsigned)grid), dim3(256), 0, st, q);
   return check_launch("moe_gemm_mxd_kernel");
 }
 template <int MR>
@@ -363,6 +372,8 @@ int32_t launch_mxd(const GemmParams& p, int grid_m, bool swiglu, hipStream_t st)
   // few rows only a few experts are live and the kernel needs every wave it can get to keep HBM busy; from about a
   // hundred rows on the activation traffic is what limits it.  (Measured at 128 experts, top-4: 16 tokens are 6 %
   // faster with one fragment, 64 tokens 8 % faster with two.)
+  if constexpr (MR == 1)
+    if (p.M <= 16) return launch_mxd_n<1, 1, true>(p, grid_m, swiglu, st);
   return p.M >= 128 ? launch_mxd_n<MR, 2>(p, grid_m, swiglu, st) : launch_mxd_n<MR, 1>(p, grid_m, swiglu, st);
 }
 

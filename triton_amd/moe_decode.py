@@ -159,7 +159,7 @@ def moe_mlp(x, logits, n_expts_act, w1, b1, w2, b2, pc1: PrecisionConfig, pc2: P
     """`routing` + gather-`matmul_ogs` (+ fused activation) + scatter-`matmul_ogs` (gate weighted, k rows summed) as one
     call: one kernel launch at decode sizes, the three calls otherwise.  Returns `[tokens, d_model]`."""
     # (with fewer than 8 routed rows the launch's fixed part, every workgroup routing the batch before its first weight
-    # byte, outweighs the two launch boundaries it saves: 41 against 33 us for one token at the gpt-oss shape)
+    # byte, outweighs the two launch boundaries it saves: 41 against 29 us for one token at the gpt-oss shape)
     if logits.shape[0] * n_expts_act >= MIN_ROWS and one_launch_reason(x, logits, n_expts_act, w1, b1, w2, b2, pc1, pc2, fused_activation) is None:
         return moe_decode_layer(x, logits, n_expts_act, w1, b1, w2, b2, pc1, pc2, fused_activation)
     from .legacy import matmul_ogs, routing
